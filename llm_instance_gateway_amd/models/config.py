@@ -21,7 +21,9 @@ class LayerSpec:
     vector), the mixer's sizes and constants, and its feed-forward (None for
     a layer without one).  'latent_attention' keeps one paged row per token
     (the normalised key/value latent followed by the shared rotated key
-    part).  `shift` says the mixer's input is blended with the previous
+    part).  'wkv' keeps a matrix state per head and the previous token's
+    input row; 'parallel' keeps paged K/V for its attention branch and a
+    matrix state per head for its recurrent branch.  `shift` says the mixer's input is blended with the previous
     token's, which costs one fp32 row of model width per sequence."""
 
     type: str
@@ -66,6 +68,10 @@ class ModelConfig:
     layer_loop: Optional[Tuple[int, int, int]] = None
     # Folder with config.json + model.safetensors ("" = random init).
     weights_path: str = ""
+    # Post-norm stacks: x <- norm(residual_alpha * x + sublayer(x)).
+    residual_alpha: float = 1.0
+    # logits <- cap * tanh(logits / cap); 0 = no cap.
+    logit_softcap: float = 0.0
 
     @property
     def is_moe(self) -> bool:
@@ -98,6 +104,11 @@ class ModelConfig:
                 total += (s.mixer["kv_heads"] // tp_size) * (s.mixer["dim"] + s.mixer["vdim"])
             elif s.type == "latent_attention":
                 total += s.mixer["kv_rank"] + s.mixer["rot_dim"]
+            elif s.type == "parallel":
+                # the attention branch caches normed keys and, as values, the
+                # keys as projected
+                left = s.mixer["left"]
+                total += (left["kv_heads"] // tp_size) * 2 * left["dim"]
         return total
 
     def state_elems_per_seq(self) -> int:
@@ -109,6 +120,12 @@ class ModelConfig:
             s = self.layer_specs[i]
             if s.type == "mingru":
                 total += s.mixer["width"]
+            elif s.type == "wkv":
+                # previous token's input row + one matrix per head
+                total += self.hidden_size + s.mixer["heads"] * s.mixer["dim"] ** 2
+            elif s.type == "parallel":
+                right = s.mixer["right"]
+                total += right["heads"] * right["dim"] * right["vdim"]
             if s.shift:
                 total += self.hidden_size
         return total

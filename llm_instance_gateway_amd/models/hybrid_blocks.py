@@ -430,3 +430,285 @@ class ScoredExpertsMLP(nn.Module):
         back = torch.empty_like(dest)
         back[order] = dest
         return ye.index_select(0, back).view(T, self.top, hidden).float().sum(dim=1).to(h.dtype)
+
+
+class NormedRotaryAttention(nn.Module):
+    """Grouped-query softmax attention whose queries and keys are RMS-normed
+    before an optional partial rotate-half rotation, with optional chunked
+    visibility (a query sees the keys of its own chunk of `chunk` positions,
+    counted from the sequence's start).
+
+      * qk_norm "row": one norm over the whole q (and k) projection with
+        weights of that size; "head": per head with one weight of size dim
+        shared by the heads; "none".
+      * rot_dims entries of every head are rotated (pairs i, i + rot_dims/2);
+        0 = no rotation.
+      * values "proj": a projection of their own; "key": the keys as
+        projected, before their norm (no value weights).
+      * v_unit_norm: every head's value is divided by its root mean square.
+      * value mixing: `forward(..., v_first=...)` blends the values with
+        those another layer computed for the same tokens, (1 - lam) v + lam
+        v_first, before they are cached; `want_v` returns this layer's.
+      * dist_bias / talk: a per-head bias by distance, added to the scaled
+        score, and a [heads, heads] matrix that mixes the heads' scores
+        before the softmax.  With either, all heads of a token are scored
+        together by the head-mixing kernel.
+
+    Projections (biases optional) are one fused GEMM in, one out; everything
+    between the GEMMs and the attention kernel is one prep kernel.  A model
+    may pass `proj` (a wider fused projection that starts with this block's
+    q | k | v columns) instead of letting the block run its own GEMM.
+    """
+
+    def __init__(
+        self, hidden: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+        eps: float, qk_norm: str = "row", rot_base: float = 10000.0, rot_dims: int = 0,
+        chunk: int = 0, values: str = "proj", v_unit_norm: bool = False, bias: bool = True,
+        dist_rows: int = 0, dist_far: float = 0.0, talk: bool = False,
+        device="cpu", dtype=torch.bfloat16,
+    ) -> None:
+        super().__init__()
+        assert heads % kv_heads == 0 and qk_norm in ("none", "row", "head")
+        assert values in ("proj", "key") and (values == "proj" or vdim == dim)
+        assert 0 <= rot_dims <= dim and rot_dims % 2 == 0
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.eps, self.chunk = float(scale), float(eps), int(chunk)
+        self.qk_norm, self.values, self.v_unit_norm = qk_norm, values, v_unit_norm
+        self.nq, self.nk = heads * dim, kv_heads * dim
+        self.nv = kv_heads * vdim if values == "proj" else 0
+        self.n_in = self.nq + self.nk + self.nv
+        s = 1.0 / math.sqrt(hidden)
+        self.w_in = _param((self.n_in, hidden), device, dtype, s)
+        self.b_in = _param((self.n_in,), device, dtype, 0.1 if bias else None)
+        self.has_bias = bias
+        nw = {"row": (self.nq, self.nk), "head": (dim, dim), "none": (0, 0)}[qk_norm]
+        self.q_norm = _param((nw[0],), device, dtype, None)
+        self.k_norm = _param((nw[1],), device, dtype, None)
+        with torch.no_grad():
+            self.q_norm.fill_(1.0)
+            self.k_norm.fill_(1.0)
+        self.w_o = _param((hidden, heads * vdim), device, dtype, 1.0 / math.sqrt(heads * vdim))
+        self.b_o = _param((hidden,), device, dtype, 0.1 if bias else None)
+        self.lam = 0.0  # value-mixing weight
+        self.dist_far = float(dist_far)
+        # fp32 whatever the activation dtype: they enter the scores
+        self.rel = (
+            nn.Parameter(torch.empty(dist_rows, heads, device=device).uniform_(-0.5, 0.5), requires_grad=False)
+            if dist_rows > 0 else None
+        )
+        self.talk = (
+            nn.Parameter(
+                torch.eye(heads, device=device) + torch.empty(heads, heads, device=device).uniform_(-0.1, 0.1),
+                requires_grad=False,
+            )
+            if talk else None
+        )
+        self.dist_bias: Optional[torch.Tensor] = None
+        self.refresh_tables()
+        self.register_buffer(
+            "inv_freq",
+            ops.rotary_inv_freq(rot_base, rot_dims, device) if rot_dims > 0 else None,
+            persistent=False,
+        )
+
+    def refresh_tables(self) -> None:
+        """Expand the bucketed distance table to one row per distance."""
+        if self.rel is not None:
+            self.dist_bias = ops.distance_bias_table(self.rel, self.dist_far)
+
+    @property
+    def mixes_heads(self) -> bool:
+        return self.rel is not None or self.talk is not None
+
+    def cache_spec(self) -> dict:
+        return {"kind": "kv", "kv_heads": self.kv_heads, "k_dim": self.dim, "v_dim": self.vdim}
+
+    def load(self, get, prefix: str) -> None:
+        names = ["q", "k"] + (["v"] if self.values == "proj" else [])
+        with torch.no_grad():
+            self.w_in.copy_(torch.cat([get(prefix + n) for n in names], dim=0))
+            if self.has_bias:
+                self.b_in.copy_(torch.cat([get(prefix + n + ".b") for n in names], dim=0))
+                self.b_o.copy_(get(prefix + "o.b"))
+            if self.qk_norm != "none":
+                self.q_norm.copy_(get(prefix + "q.norm"))
+                self.k_norm.copy_(get(prefix + "k.norm"))
+            self.w_o.copy_(get(prefix + "o"))
+            if self.rel is not None:
+                self.rel.copy_(get(prefix + "rel").float())
+            if self.talk is not None:
+                self.talk.copy_(get(prefix + "talk").float())
+        self.refresh_tables()
+
+    def forward(self, h, positions, cache, meta, v_first=None, want_v=False, proj=None):
+        k_cache, v_cache = cache
+        if proj is None:
+            proj = F.linear(h, self.w_in, self.b_in if self.has_bias else None)
+        q, v_out = ops.qkv_norm_rope_cache(
+            proj, self.heads, self.kv_heads, self.dim, self.vdim, self.qk_norm,
+            self.q_norm, self.k_norm, self.eps, self.inv_freq, positions, k_cache, v_cache,
+            meta.slot_mapping, v_source=self.values, v_unit_norm=self.v_unit_norm,
+            v_first=v_first, lam=self.lam, want_v=want_v,
+        )
+        if self.mixes_heads:
+            o = ops.paged_attention_mixed_heads(
+                q, k_cache, v_cache, meta.seq_block_tables, meta.tok_seq, positions,
+                self.scale, self.heads, dist_bias=self.dist_bias, talk=self.talk,
+                chunk=self.chunk,
+            )
+        else:
+            o = self._attend(q, positions, k_cache, v_cache, meta)
+        y = F.linear(o, self.w_o, self.b_o if self.has_bias else None)
+        return (y, v_out) if want_v else y
+
+    def _attend(self, q, positions, k_cache, v_cache, meta):
+        np_, rows = meta.num_prefill_tokens, q.shape[0]
+        if (
+            np_ > 0
+            and meta.prefill_tile_seq is not None
+            and ops.tiled_prefill_supported(q.dtype, self.dim, self.vdim, q.is_cuda)
+        ):
+            # prompt portions on MFMA tiles, the step's single tokens (and
+            # pad rows) through the any-shape kernel
+            o = torch.empty(rows, self.heads * self.vdim, dtype=q.dtype, device=q.device)
+            ops.paged_attention_prefill_tiles(
+                q[:np_], k_cache, v_cache, meta.prefill_block_tables,
+                meta.prefill_query_start_locs, meta.prefill_context_lens,
+                meta.prefill_tile_seq, meta.prefill_tile_qstart, self.scale, self.heads,
+                out=o[:np_], chunk=self.chunk,
+            )
+            if rows > np_:
+                ops.paged_attention_general(
+                    q[np_:], k_cache, v_cache, meta.seq_block_tables, meta.tok_seq[np_:],
+                    positions[np_:], self.scale, self.heads, out=o[np_:], chunk=self.chunk,
+                )
+            return o
+        return ops.paged_attention_general(
+            q, k_cache, v_cache, meta.seq_block_tables, meta.tok_seq, positions,
+            self.scale, self.heads, chunk=self.chunk,
+        )
+
+
+class MatrixStateMixer(nn.Module):
+    """Recurrent mixers that carry one [dim, vdim] fp32 matrix per head and
+    sequence (slot pool), scanned token by token by `ops.matrix_state_scan`.
+
+    kind "wkv": every projection reads its own blend of the input with the
+    previous token's (`ops.token_shift_mix`, five blends, one more state row
+    per sequence); per-channel per-token decay w = exp(-exp(W_w2 tanh(W_w1 .)
+    + w0)) from a low-rank pair; the current token enters the output through
+    a bonus u instead of the state; every head's output is divided by its
+    root mean square, then times a weight, times silu(gate).
+
+    kind "decay": q, k, v pass through silu, one constant decay per head, the
+    output reads the updated state; the concatenated heads are RMS-normed
+    together with a weight and multiplied by sigmoid(gate).
+
+    A model may hand "decay" a wider fused projection (`proj`, columns q | k
+    | v | gate first) instead of letting the block run its own GEMM.
+    """
+
+    def __init__(
+        self, hidden: int, kind: str, heads: int, dim: int, vdim: int, eps: float,
+        decay=None, decay_rank: int = 0, device="cpu", dtype=torch.bfloat16,
+    ) -> None:
+        super().__init__()
+        assert kind in ("wkv", "decay")
+        self.kind, self.heads, self.dim, self.vdim, self.eps = kind, heads, dim, vdim, float(eps)
+        self.hidden = hidden
+        nk, nv = heads * dim, heads * vdim
+        self.nk, self.nv = nk, nv
+        s = 1.0 / math.sqrt(hidden)
+        if kind == "wkv":
+            assert vdim == dim
+            # blends in the order r, k, v, gate, decay
+            self.mu = _param((5, hidden), device, dtype, None)
+            with torch.no_grad():
+                self.mu.uniform_(0.0, 1.0)
+            # pre-transposed for one batched GEMM: [4, hidden, heads*dim]
+            self.w_rkvg = _param((4, hidden, nk), device, dtype, s)
+            self.w_d1 = _param((decay_rank, hidden), device, dtype, s)
+            # the decay's second projection, its offset and the bonus enter
+            # the recurrence: fp32
+            self.w_d2 = nn.Parameter(
+                torch.empty(nk, decay_rank, device=device).uniform_(-0.1, 0.1), requires_grad=False
+            )
+            self.d0 = nn.Parameter(torch.empty(nk, device=device).uniform_(-1.0, 0.5), requires_grad=False)
+            self.bonus = nn.Parameter(torch.empty(nk, device=device).uniform_(-0.5, 0.5), requires_grad=False)
+            self.head_decay = None
+        else:
+            # rows: q | k | v | gate
+            self.w_in = _param((2 * nk + 2 * nv, hidden), device, dtype, s)
+            self.head_decay = nn.Parameter(
+                torch.tensor([float(d) for d in decay], dtype=torch.float32, device=device),
+                requires_grad=False,
+            )
+            assert self.head_decay.shape == (heads,)
+        self.norm = _param((nv,), device, dtype, None)
+        with torch.no_grad():
+            self.norm.fill_(1.0)
+        self.w_o = _param((hidden, nv), device, dtype, 1.0 / math.sqrt(nv))
+
+    def cache_spec(self):
+        mat = {"kind": "state", "width": ops.matrix_state_width(self.heads, self.dim, self.vdim)}
+        if self.kind == "wkv":
+            return [{"kind": "state", "width": self.hidden}, mat]
+        return mat
+
+    def load(self, get, prefix: str) -> None:
+        with torch.no_grad():
+            if self.kind == "wkv":
+                self.mu.copy_(torch.stack([get(prefix + "mu." + n) for n in "rkvgw"], dim=0))
+                self.w_rkvg.copy_(torch.stack([get(prefix + n).t() for n in "rkvg"], dim=0))
+                self.w_d1.copy_(get(prefix + "w1"))
+                self.w_d2.copy_(get(prefix + "w2").float())
+                self.d0.copy_(get(prefix + "w0").float())
+                self.bonus.copy_(get(prefix + "u").float().reshape(-1))
+            else:
+                self.w_in.copy_(torch.cat([get(prefix + n) for n in "qkvg"], dim=0))
+            self.norm.copy_(get(prefix + "norm"))
+            self.w_o.copy_(get(prefix + "o"))
+
+    def forward(self, x, h, cache, meta, proj=None):
+        """x: the fp32 rows (token shift reads them), h: the same in the
+        activation dtype."""
+        seg = (meta.seg_start, meta.seg_len, meta.seg_slot, meta.seg_fresh)
+        if self.kind == "wkv":
+            shift_state, mat_state = cache
+            mixes = ops.token_shift_mix(x, self.mu, shift_state, meta.tok_seq, *seg)
+            rkvg = torch.bmm(mixes[:4], self.w_rkvg)  # [4, R, heads*dim]
+            low = ops.tanh_act(F.linear(mixes[4], self.w_d1))
+            decay_pre = F.linear(low.float(), self.w_d2, self.d0)  # fp32
+            o = ops.matrix_state_scan(
+                rkvg[0], rkvg[1], rkvg[2], mat_state, *seg, self.heads, self.dim, self.vdim,
+                decay_pre=decay_pre, bonus=self.bonus,
+            )
+            g = ops.group_rms_norm_gate(o, rkvg[3], self.norm, self.vdim, "silu", self.eps)
+        else:
+            (mat_state,) = cache
+            if proj is None:
+                proj = F.linear(h, self.w_in)
+            a, b, c = self.nk, 2 * self.nk, 2 * self.nk + self.nv
+            o = ops.matrix_state_scan(
+                proj[:, :a], proj[:, a:b], proj[:, b:c], mat_state, *seg, self.heads,
+                self.dim, self.vdim, head_decay=self.head_decay, act_silu=True,
+            )
+            g = ops.group_rms_norm_gate(o, proj[:, c : c + self.nv], self.norm, self.nv, "sigmoid", self.eps)
+        return F.linear(g, self.w_o)
+
+
+class GeluMLP(nn.Module):
+    """down(gelu(up h)) with the exact (erf) gelu."""
+
+    def __init__(self, hidden: int, ff: int, device="cpu", dtype=torch.bfloat16) -> None:
+        super().__init__()
+        self.w_up = _param((ff, hidden), device, dtype, 1.0 / math.sqrt(hidden))
+        self.w_down = _param((hidden, ff), device, dtype, 1.0 / math.sqrt(ff))
+
+    def load(self, get, prefix: str) -> None:
+        with torch.no_grad():
+            self.w_up.copy_(get(prefix + "up"))
+            self.w_down.copy_(get(prefix + "down"))
+
+    def forward(self, h, meta=None):
+        return _mm(ops.gelu_erf(_mm(h, self.w_up)), self.w_down)

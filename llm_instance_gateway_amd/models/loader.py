@@ -30,6 +30,14 @@ _DTYPES = {
 }
 
 
+def read_safetensors_shapes(path: str) -> Dict[str, list]:
+    """Tensor name -> shape from the header alone (no tensor data is read)."""
+    with open(path, "rb") as f:
+        (hlen,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(hlen).decode("utf-8"))
+    return {k: list(v["shape"]) for k, v in header.items() if k != "__metadata__"}
+
+
 def read_safetensors(path: str) -> Dict[str, torch.Tensor]:
     with open(path, "rb") as f:
         mm = mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_COPY)

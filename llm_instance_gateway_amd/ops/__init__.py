@@ -481,13 +481,15 @@ def paged_attention_general(
     q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float,
     num_heads: int, gate=None, temp_coef: float = 0.0, temp_every: float = 1.0,
     out: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
+    chunk: int = 0,
 ) -> torch.Tensor:
     """Causal paged attention for any key/value head sizes; token r of the
     flat batch attends keys 0..positions[r] of sequence tok_seq[r].  Optional
     query temperature 1 + coef*ln(floor((p+1)/every)+1), sigmoid output gate
     and per-head softmax sink (fp32 [heads]: exp(sink) joins the denominator).
     q/gate may be column-block views with a row stride; v_cache may be a view
-    of the leading entries of k_cache's rows (a latent cache)."""
+    of the leading entries of k_cache's rows (a latent cache).  chunk > 0:
+    only keys of the query's own chunk, floor(j/chunk) == floor(p/chunk)."""
     if _use_hybrid(q):
         nb, G, bs, D = k_cache.shape
         Dv = v_cache.shape[-1]
@@ -511,12 +513,12 @@ def paged_attention_general(
             _ptr(block_tables), block_tables.shape[1], _ptr(tok_seq),
             _ptr(positions), _ptr(gate), 0 if gate is None else gate.stride(0),
             _ptr(sink), float(scale), float(temp_coef), ev, ev_int, R, num_heads,
-            G, D, Dv, v_row, bs, _is_f32(q), _stream(),
+            G, D, Dv, v_row, bs, int(chunk), _is_f32(q), _stream(),
         )
         return out
     res = torch_ref.paged_attention_general(
         q, k_cache, v_cache, block_tables, tok_seq, positions, scale, num_heads,
-        gate, temp_coef, temp_every, sink,
+        gate, temp_coef, temp_every, sink, chunk,
     )
     if out is not None:
         out.copy_(res)
@@ -578,15 +580,15 @@ def paged_attention_prefill_tiles(
     q, k_cache, v_cache, block_tables, query_start_locs, context_lens, tile_seq,
     tile_qstart, scale: float, num_heads: int, gate=None, temp_coef: float = 0.0,
     temp_every: float = 1.0, out: Optional[torch.Tensor] = None,
-    sink: Optional[torch.Tensor] = None,
+    sink: Optional[torch.Tensor] = None, chunk: int = 0,
 ) -> torch.Tensor:
     """Prompt-partition attention on MFMA tiles for any head sizes the kernel
     takes (`tiled_prefill_supported`): q [Tp, H*D] (strided view allowed) are
     the rows of the step's prompt portions, laid out by query_start_locs;
     context_lens count each sequence's tokens after this step; tile_seq /
     tile_qstart name the 64-row query tiles.  Temperature, sigmoid gate and
-    softmax sink are fused; v_cache may view the head of k_cache's rows.  GPU
-    only."""
+    softmax sink are fused; v_cache may view the head of k_cache's rows; chunk
+    > 0 restricts every row to the keys of its own chunk.  GPU only."""
     nb, G, bs, D = k_cache.shape
     Dv = v_cache.shape[-1]
     v_row = _value_row_stride(v_cache)
@@ -610,7 +612,7 @@ def paged_attention_prefill_tiles(
         _ptr(tile_qstart), _ptr(query_start_locs), _ptr(context_lens),
         _ptr(block_tables), float(scale), float(temp_coef), ev, ev_int,
         tile_seq.shape[0], num_heads, G, D, Dv, v_row, bs, block_tables.shape[1],
-        _stream(),
+        int(chunk), _stream(),
     )
     if rc != 0:
         raise RuntimeError("paged_attention_prefill_tiles: shape or alignment not served")
@@ -832,3 +834,286 @@ def scale_gather_rows(x: torch.Tensor, idx: torch.Tensor, w: torch.Tensor) -> to
         )
         return out
     return torch_ref.scale_gather_rows(x, idx, w)
+
+
+# -- post-norm residual, normed/rotated attention inputs, chunked and
+# -- head-mixed attention, matrix-state recurrences ----------------------------------
+
+def scaled_add_rms_norm(
+    x: torch.Tensor, alpha: float, w: torch.Tensor, eps: float,
+    y1: Optional[torch.Tensor] = None, s1: float = 1.0,
+    y2: Optional[torch.Tensor] = None, s2: float = 1.0,
+):
+    """Norm after the sum on the fp32 residual x [R, H], in place:
+    x <- rms(alpha * x + s1 * y1 + s2 * y2) * w.  Returns (x, x rounded to
+    w's dtype), the second being the next sub-layer's GEMM input.  Without y1
+    the rows are only normed and x stays as it is."""
+    assert x.dtype == torch.float32 and (y2 is None or y1 is not None)
+    if _use_hybrid(x):
+        R, H = x.shape
+        assert x.is_contiguous() and w.shape == (H,)
+        for y in (y1, y2):
+            assert y is None or (y.shape == x.shape and y.is_contiguous() and y.dtype == w.dtype)
+        h = torch.empty(R, H, dtype=w.dtype, device=x.device)
+        _hl().lig_scaled_add_rms_norm(
+            _ptr(x), _ptr(h), _ptr(y1), _ptr(y2), _ptr(w), float(alpha), float(s1),
+            float(s2), float(eps), R, H, _is_f32(w), _stream(),
+        )
+        return x, h
+    return torch_ref.scaled_add_rms_norm(x, alpha, w, eps, y1, s1, y2, s2, w.dtype)
+
+
+_QK_NORM_MODES = {"none": 0, "row": 1, "head": 2}
+
+
+def qkv_norm_rope_cache(
+    proj, heads: int, kv_heads: int, dim: int, vdim: int, qk_norm: str, w_q, w_k,
+    eps: float, inv_freq, positions, k_cache, v_cache, slot_mapping,
+    v_source: str = "proj", v_unit_norm: bool = False, v_first=None, lam: float = 0.0,
+    want_v: bool = False,
+):
+    """Everything between the fused input projection and the attention
+    kernel, one pass per token row of proj = [q | k | v] (or [q | k] with
+    v_source "key": the values are the keys as projected).
+
+    qk_norm "row": RMS norm over all of q (and of k) with weights of that
+    size; "head": per head, one weight of size dim shared by the heads;
+    "none".  Then rotate-half rotation of the first 2*len(inv_freq) entries
+    of every q and k head (inv_freq None: no rotation).  Values: optionally
+    divided per head by their root mean square, optionally blended with
+    v_first (fp32 [R, kv_heads*vdim]) as (1 - lam) v + lam v_first.  Keys and
+    values go to the paged caches at slot_mapping; returns (q [R, heads*dim]
+    contiguous, the values as cached in fp32 if want_v else None)."""
+    mode = _QK_NORM_MODES[qk_norm]
+    from_key = v_source == "key"
+    assert v_source in ("proj", "key") and (not from_key or vdim == dim)
+    if _use_hybrid(proj):
+        R = proj.shape[0]
+        nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
+        assert proj.stride(1) == 1 and proj.shape[1] >= nq + nk + (0 if from_key else nv)
+        nb, G, bs, D = k_cache.shape
+        assert G == kv_heads and D == dim and v_cache.shape == (nb, G, bs, vdim)
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == proj.dtype
+        assert positions.dtype == torch.int64 and slot_mapping.dtype == torch.int64
+        if mode == 1:
+            assert w_q.shape == (nq,) and w_k.shape == (nk,)
+        elif mode == 2:
+            assert w_q.shape == (dim,) and w_k.shape == (dim,)
+        nf = 0
+        if inv_freq is not None and inv_freq.numel() > 0:
+            nf = inv_freq.shape[0]
+            assert inv_freq.dtype == torch.float32 and 2 * nf <= dim
+        if v_first is not None:
+            assert v_first.dtype == torch.float32 and v_first.shape == (R, nv) and v_first.is_contiguous()
+        q_out = torch.empty(R, nq, dtype=proj.dtype, device=proj.device)
+        v_out = torch.empty(R, nv, dtype=torch.float32, device=proj.device) if want_v else None
+        _hl().lig_qkv_norm_rope_cache(
+            _ptr(q_out), _ptr(v_out), _ptr(proj), proj.stride(0), _ptr(w_q) if mode else None,
+            _ptr(w_k) if mode else None, _ptr(inv_freq) if nf else None, nf, _ptr(positions),
+            _ptr(v_first), float(lam), _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping),
+            float(eps), R, heads, kv_heads, dim, vdim, mode, int(from_key),
+            int(bool(v_unit_norm)), bs, _is_f32(proj), _stream(),
+        )
+        return q_out, v_out
+    return torch_ref.qkv_norm_rope_cache(
+        proj, heads, kv_heads, dim, vdim, qk_norm, w_q, w_k, eps, inv_freq, positions,
+        v_source, v_unit_norm, v_first, lam, want_v, k_cache, v_cache, slot_mapping,
+    )
+
+
+def distance_bias_table(rel: torch.Tensor, far: float) -> torch.Tensor:
+    """Expand a bucketed distance table rel [rows, H] into one row per
+    distance, fp32 [N, H]: distance n < rows/2 reads row n, larger distances
+    row rows/2 + floor(ln(n / (rows/2)) / ln(far / (rows/2)) * (rows - rows/2)),
+    capped at the last row.  The table stops at the first distance that
+    reaches the last row; all larger distances read that entry."""
+    import math
+
+    rows = rel.shape[0]
+    half = rows // 2
+    idx = []
+    n = 0
+    while True:
+        if n < half:
+            b = n
+        else:
+            b = min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (rows - half))))
+        idx.append(b)
+        if b == rows - 1 or n > (1 << 22):
+            break
+        n += 1
+    return rel.float()[torch.tensor(idx, dtype=torch.long, device=rel.device)].contiguous()
+
+
+def paged_attention_mixed_heads(
+    q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float, num_heads: int,
+    dist_bias: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None,
+    chunk: int = 0, out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Causal paged attention whose heads are not independent: token r sees
+    keys j <= p = positions[r] of its sequence inside its chunk
+    (floor(j/chunk) == floor(p/chunk); chunk 0: all); the scaled score of
+    head g gets dist_bias[min(p - j, N - 1), g] (fp32 [N, H]) added, then the
+    heads' scores are mixed, s_h <- sum_g talk[h, g] s_g (fp32 [H, H]),
+    before an ordinary softmax per head.  One workgroup per token holds all
+    heads' scores of a key tile.  Any head sizes, bf16 or fp32 storage."""
+    nb, G, bs, D = k_cache.shape
+    Dv = v_cache.shape[-1]
+    R = q.shape[0]
+    if _use_hybrid(q):
+        assert q.shape[1] == num_heads * D and q.stride(1) == 1 and num_heads % G == 0
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == q.dtype
+        assert block_tables.dtype == torch.int32 and tok_seq.dtype == torch.int32
+        assert positions.dtype == torch.int64 and block_tables.is_contiguous()
+        for t, shp in ((dist_bias, None), (talk, (num_heads, num_heads))):
+            if t is not None:
+                assert t.dtype == torch.float32 and t.is_contiguous()
+                assert shp is None or t.shape == shp
+        if dist_bias is not None:
+            assert dist_bias.dim() == 2 and dist_bias.shape[1] == num_heads
+        if out is None:
+            out = torch.empty(R, num_heads * Dv, dtype=q.dtype, device=q.device)
+        assert out.shape == (R, num_heads * Dv) and out.is_contiguous() and out.dtype == q.dtype
+        rc = _hl().lig_paged_attention_mixed_heads(
+            _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+            block_tables.shape[1], _ptr(tok_seq), _ptr(positions), _ptr(dist_bias),
+            0 if dist_bias is None else dist_bias.shape[0], _ptr(talk), float(scale),
+            int(chunk), R, num_heads, G, D, Dv, bs, _is_f32(q), _stream(),
+        )
+        if rc != 0:
+            raise RuntimeError("paged_attention_mixed_heads: more than 64 heads or values wider than 256")
+        return out
+    rel = dist_bias
+    res = torch_ref.paged_attention_chunked(
+        q, k_cache, v_cache, block_tables, tok_seq, positions, scale, num_heads, chunk,
+        talk=talk, dist_bias=rel,
+    )
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
+
+
+def token_shift_mix(x, mu, state, tok_seq, seg_start, seg_len, seg_slot, seg_fresh) -> torch.Tensor:
+    """Several blends of every row with the row before it, from one pass:
+    out[m] = x + (x_prev - x) * mu[m], x fp32 [R, W], mu [n, W] -> [n, R, W]
+    in mu's dtype.  Ahead of a segment's first row stands the sequence's
+    state row (zeros when the sequence starts here); the state [slots, W]
+    fp32 then takes the segment's last row.  Rows of no segment are zero."""
+    assert x.dtype == torch.float32 and state.dtype == torch.float32
+    if _use_hybrid(x):
+        R, W = x.shape
+        n = mu.shape[0]
+        assert x.is_contiguous() and mu.is_contiguous() and mu.shape == (n, W)
+        assert state.is_contiguous() and state.shape[1] == W
+        out = torch.empty(n, R, W, dtype=mu.dtype, device=x.device)
+        _hl().lig_token_shift_mix(
+            _ptr(out), _ptr(x), _ptr(mu), _ptr(state), _ptr(tok_seq), _ptr(seg_start),
+            _ptr(seg_len), _ptr(seg_slot), _ptr(seg_fresh), n, R, W, _is_f32(mu), _stream(),
+        )
+        return out
+    return torch_ref.token_shift_mix(x, mu, state, seg_start, seg_len, seg_slot, seg_fresh, mu.dtype)
+
+
+MATRIX_STATE_KEY_SPLIT = 4
+
+
+def matrix_state_width(heads: int, dim: int, vdim: int) -> int:
+    """fp32 entries of one sequence's matrix state: the scan kernel splits a
+    head's key channels over four lanes and keeps the state in the order its
+    threads hold it, key channels padded to a multiple of four."""
+    k = MATRIX_STATE_KEY_SPLIT
+    return heads * ((dim + k - 1) // k) * k * vdim
+
+
+def matrix_state_scan(
+    q, k, v, state, seg_start, seg_len, seg_slot, seg_fresh, heads: int, dim: int,
+    vdim: int, decay_pre=None, head_decay=None, bonus=None, act_silu: bool = False,
+) -> torch.Tensor:
+    """Linear recurrences with one [dim, vdim] fp32 state matrix S per head,
+    over the segments of the flat batch; q, k [R, heads*dim] and v
+    [R, heads*vdim] may be column-block views.
+
+    With `bonus` u (fp32 [heads*dim]) and decay_pre (fp32 [R, heads*dim]):
+        o_t = (S + diag(u) k_t v_t^T)^T q_t;  S <- diag(w_t) S + k_t v_t^T,
+        w_t = exp(-exp(decay_pre_t))
+    With head_decay d (fp32 [heads]):
+        S <- d_h S + k_t v_t^T;  o_t = S^T q_t
+    act_silu applies silu to q, k, v on the way in.  state [slots,
+    matrix_state_width] is read unless the segment starts its sequence and
+    written back; its layout is private to the implementation.  Returns fp32
+    [R, heads*vdim]; rows of no segment are zero."""
+    assert (bonus is None) == (decay_pre is None) and (bonus is None) != (head_decay is None)
+    assert state.dtype == torch.float32
+    if _use_hybrid(q):
+        R = q.shape[0]
+        assert q.shape[1] == heads * dim and k.shape[1] == heads * dim and v.shape[1] == heads * vdim
+        assert q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1
+        assert q.dtype == k.dtype == v.dtype
+        assert state.is_contiguous() and state.shape[1] == matrix_state_width(heads, dim, vdim)
+        for t, n in ((decay_pre, R * heads * dim), (bonus, heads * dim), (head_decay, heads)):
+            if t is not None:
+                assert t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n
+        S = seg_start.shape[0]
+        out = torch.zeros(R, heads * vdim, dtype=torch.float32, device=q.device)
+        rc = _hl().lig_matrix_state_scan(
+            _ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
+            _ptr(decay_pre), _ptr(head_decay), _ptr(bonus), _ptr(state), state.stride(0),
+            _ptr(seg_start), _ptr(seg_len), _ptr(seg_slot), _ptr(seg_fresh), S, heads, dim,
+            vdim, int(bool(act_silu)), _is_f32(q), _stream(),
+        )
+        if rc != 0:
+            raise RuntimeError("matrix_state_scan: keys or values wider than 256 per head")
+        return out
+    return torch_ref.matrix_state_scan(
+        q, k, v, state, seg_start, seg_len, seg_slot, seg_fresh, heads, dim, vdim,
+        decay_pre, head_decay, bonus, act_silu,
+    )
+
+
+def group_rms_norm_gate(o, gate, w, group: int, gate_act: str, eps: float) -> torch.Tensor:
+    """o fp32 [R, C]: every `group` consecutive entries are divided by their
+    root mean square (group == C: the whole row), then times w [C], times
+    silu(gate) or sigmoid(gate); gate [R, C] may be a column-block view.
+    Result in w's dtype."""
+    assert o.dtype == torch.float32 and gate_act in ("silu", "sigmoid")
+    R, C = o.shape
+    assert C % group == 0 and gate.shape == (R, C) and w.shape == (C,)
+    if _use_hybrid(o):
+        assert o.is_contiguous() and gate.stride(1) == 1 and gate.dtype == w.dtype
+        out = torch.empty(R, C, dtype=w.dtype, device=o.device)
+        _hl().lig_group_rms_norm_gate(
+            _ptr(out), _ptr(o), _ptr(gate), gate.stride(0), _ptr(w), int(group),
+            1 if gate_act == "silu" else 0, float(eps), R, C, _is_f32(w), _stream(),
+        )
+        return out
+    return torch_ref.group_rms_norm_gate(o, gate, w, group, gate_act, eps, w.dtype)
+
+
+def gelu_erf(x: torch.Tensor) -> torch.Tensor:
+    """The exact gelu, 0.5 z (1 + erf(z / sqrt 2))."""
+    if _use_hybrid(x):
+        assert x.is_contiguous()
+        out = torch.empty_like(x)
+        _hl().lig_gelu_erf(_ptr(out), _ptr(x), x.numel(), _is_f32(x), _stream())
+        return out
+    return torch_ref.gelu_erf(x)
+
+
+def tanh_act(x: torch.Tensor) -> torch.Tensor:
+    if _use_hybrid(x):
+        assert x.is_contiguous()
+        out = torch.empty_like(x)
+        _hl().lig_tanh_act(_ptr(out), _ptr(x), x.numel(), _is_f32(x), _stream())
+        return out
+    return torch_ref.tanh_act(x)
+
+
+def tanh_softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap * tanh(x / cap) in place on fp32 logits."""
+    assert x.dtype == torch.float32
+    if _use_hybrid(x):
+        assert x.is_contiguous()
+        _hl().lig_tanh_softcap(_ptr(x), float(cap), x.numel(), _stream())
+        return x
+    return torch_ref.tanh_softcap(x, cap)

@@ -19,6 +19,10 @@
 // key with that (unscaled) score and no value, counted once per row.  The
 // running max starts at the sink and the running sum at one.
 //
+// chunk > 0 restricts a query at position p to the keys of its own chunk,
+// floor(j / chunk) == floor(p / chunk), chunks counted from position 0 of the
+// sequence.
+//
 // Cache layout: K [blocks, G, BS, D], V [blocks, G, BS, v_row] of which the
 // first Dv entries of a row are the value (v_row == Dv for a cache of its
 // own; a latent cache passes the key rows themselves, v_row == D).
@@ -37,7 +41,7 @@ __global__ void paged_attention_general_kernel(
     const int64_t* __restrict__ positions,  // [R]
     const T* __restrict__ gate, long gate_stride, const float* __restrict__ sink,
     float scale, float temp_coef, float temp_every, int temp_every_int, int H,
-    int G, int D, int Dv, int v_row, int BS) {
+    int G, int D, int Dv, int v_row, int BS, int chunk) {
   extern __shared__ __align__(16) float smem[];
   float* q_s = smem;                       // [D], padded to an even count
   float* p_s = smem + ((D + 1) & ~1);      // [64]
@@ -77,7 +81,9 @@ __global__ void paged_attention_general_kernel(
 #pragma unroll
   for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) acc[i] = 0.f;
 
-  for (int j0 = 0; j0 < ctx; j0 += WAVE_SIZE) {
+  // chunked visibility: the walk starts at the first key of the query's chunk
+  const int first_key = chunk > 0 ? (int)(pos / chunk) * chunk : 0;
+  for (int j0 = first_key; j0 < ctx; j0 += WAVE_SIZE) {
     const int j = j0 + lane;
     const bool valid = j < ctx;
     float score = -INFINITY;
@@ -286,7 +292,7 @@ void lig_paged_attention_general(
     const int* tok_seq, const int64_t* positions, const void* gate,
     long gate_stride, const float* sink, float scale, float temp_coef,
     float temp_every, int temp_every_int, int R, int H, int G, int D, int Dv,
-    int v_row, int BS, int is_f32, hipStream_t s) {
+    int v_row, int BS, int chunk, int is_f32, hipStream_t s) {
   if (R <= 0) return;
   dim3 grid(R, H), block(WAVE_SIZE);
   const size_t smem = (size_t)(((D + 1) & ~1) + WAVE_SIZE) * sizeof(float) + WAVE_SIZE * sizeof(long);
@@ -297,7 +303,7 @@ void lig_paged_attention_general(
                      (const T*)k_cache, (const T*)v_cache, block_tables,        \
                      max_blocks, tok_seq, positions, (const T*)gate,            \
                      gate_stride, sink, scale, temp_coef, temp_every,           \
-                     temp_every_int, H, G, D, Dv, v_row, BS)
+                     temp_every_int, H, G, D, Dv, v_row, BS, chunk)
   if (is_f32) {
     if (vec) LIG_LAUNCH_ATT(float, true); else LIG_LAUNCH_ATT(float, false);
   } else {

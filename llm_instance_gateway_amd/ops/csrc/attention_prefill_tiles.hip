@@ -18,7 +18,8 @@
 // the epilogue.  K and V are staged separately since their rows differ in
 // length.  An optional per-head sink starts every row's running max at
 // sink_h and its running sum at one (a key with that unscaled score and no
-// value).  A value row is the first Dv entries of a cache row of v_row
+// value).  chunk > 0 restricts a row at position p to keys j with
+// floor(j / chunk) == floor(p / chunk).  A value row is the first Dv entries of a cache row of v_row
 // entries, so a latent cache can pass its key rows as values.
 
 #include "elem_types.h"
@@ -42,7 +43,7 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
     const int* __restrict__ context_lens,      // [S] after this step's tokens
     const int* __restrict__ block_tables, float scale, float temp_coef,
     float temp_every, int temp_every_int, int num_q_heads, int num_kv_heads,
-    int D, int Dv, int v_row, int block_size, int max_blocks) {
+    int D, int Dv, int v_row, int block_size, int max_blocks, int chunk) {
   constexpr int DB = DVP / 16;
   constexpr int KB = DKP / 32;
 
@@ -110,7 +111,13 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
 
   const int kv_end_tile = min(ctx, ctx - n + qt + PT_TQ);
 
-  for (int kv0 = 0; kv0 < kv_end_tile; kv0 += PT_KVBLK) {
+  // chunked visibility: a row at position p sees keys from floor(p / chunk)
+  // * chunk on; the tile's walk starts at its first row's chunk
+  const int qpos0 = ctx - n + qt;
+  const int kv_begin = chunk > 0 ? (qpos0 / chunk) * chunk : 0;
+  const int key_lo = (chunk > 0 && row_valid) ? (qpos / chunk) * chunk : 0;
+
+  for (int kv0 = kv_begin; kv0 < kv_end_tile; kv0 += PT_KVBLK) {
     // ---- staging: K rows [32][DKP], V transposed [DVP][32]; zero padding ----
     for (int c = tid; c < PT_KVBLK * (DKP / 8); c += 256) {
       const int row = c / (DKP / 8);
@@ -171,7 +178,7 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
       for (int r = 0; r < 4; ++r) {
         const int key = kv0 + kt * 16 + lg * 4 + r;
         float v = acc_s[kt][r] * row_scale;
-        if (!row_valid || key > qpos || key >= ctx) v = -INFINITY;
+        if (!row_valid || key > qpos || key >= ctx || key < key_lo) v = -INFINITY;
         sc[kt * 4 + r] = v;
         rowmax = fmaxf(rowmax, v);
       }
@@ -265,7 +272,7 @@ extern "C" int lig_paged_attention_prefill_tiles(
     const int* context_lens, const int* block_tables, float scale,
     float temp_coef, float temp_every, int temp_every_int, int ntiles,
     int num_q_heads, int num_kv_heads, int D, int Dv, int v_row, int block_size,
-    int max_blocks, hipStream_t stream) {
+    int max_blocks, int chunk, hipStream_t stream) {
   if (D % 8 != 0 || Dv % 8 != 0 || D > 128 || Dv > 128 || D <= 0 || Dv <= 0 ||
       v_row % 8 != 0 || v_row < Dv ||
       q_stride % 8 != 0 || !aligned16(q) || !aligned16(k_cache) ||
@@ -283,7 +290,7 @@ extern "C" int lig_paged_attention_prefill_tiles(
                      query_start_locs,                                        \
                      context_lens, block_tables, scale, temp_coef, temp_every, \
                      temp_every_int, num_q_heads, num_kv_heads, D, Dv, v_row, \
-                     block_size, max_blocks)
+                     block_size, max_blocks, chunk)
   const int dkp = D <= 32 ? 32 : (D <= 64 ? 64 : 128);
   const int dvp = Dv <= 32 ? 32 : (Dv <= 64 ? 64 : 128);
   if (dkp == 32 && dvp == 32) LAUNCH_PT(32, 32);

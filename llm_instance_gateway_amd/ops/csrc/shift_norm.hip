@@ -356,3 +356,57 @@ void lig_residual_add(float* x, const void* a, const void* b, long n, int is_f32
 }
 
 }  // extern "C"
+
+// Several blends of a row with the row before it in one pass over the fp32
+// rows: out[m][r] = x[r] + (x_prev - x[r]) * mu[m].  Ahead of a segment's
+// first row stands the sequence's state row (zeros when the sequence starts
+// here).  The workgroup of a segment's FIRST row is the only one that touches
+// the state: it reads it, and then stores the segment's last row there, so
+// no other workgroup races with it.  Rows of no segment come out zero.
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_mix_kernel(
+    T* __restrict__ out, const float* __restrict__ x, const T* __restrict__ mu,
+    float* __restrict__ state, const int* __restrict__ tok_seq,
+    const int* __restrict__ seg_start, const int* __restrict__ seg_len,
+    const int* __restrict__ seg_slot, const int* __restrict__ seg_fresh,
+    int n_mix, int R, int W) {
+  const long r = blockIdx.x;
+  const int seq = tok_seq[r];
+  if (seq < 0) {
+    for (int m = 0; m < n_mix; ++m)
+      for (int c = threadIdx.x; c < W; c += blockDim.x)
+        st(out + ((long)m * R + r) * W + c, 0.f);
+    return;
+  }
+  const int s0 = seg_start[seq];
+  const bool first = r == s0;
+  const float* prev = nullptr;
+  float* srow = state + (long)seg_slot[seq] * W;
+  if (!first) prev = x + (r - 1) * W;
+  else if (!seg_fresh[seq]) prev = srow;
+  const float* last = x + ((long)s0 + seg_len[seq] - 1) * W;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float cur = x[r * W + c];
+    const float d = (prev != nullptr ? prev[c] : 0.f) - cur;
+    for (int m = 0; m < n_mix; ++m)
+      st(out + ((long)m * R + r) * W + c, cur + d * ld(mu + (long)m * W + c));
+    if (first) srow[c] = last[c];  // after this thread's own read of srow[c]
+  }
+}
+
+extern "C" void lig_token_shift_mix(void* out, const float* x, const void* mu,
+                                    float* state, const int* tok_seq,
+                                    const int* seg_start, const int* seg_len,
+                                    const int* seg_slot, const int* seg_fresh,
+                                    int n_mix, int R, int W, int is_f32,
+                                    hipStream_t s) {
+  if (R <= 0 || W <= 0) return;
+  if (is_f32)
+    hipLaunchKernelGGL(token_shift_mix_kernel<float>, dim3(R), dim3(256), 0, s,
+                       (float*)out, x, (const float*)mu, state, tok_seq, seg_start,
+                       seg_len, seg_slot, seg_fresh, n_mix, R, W);
+  else
+    hipLaunchKernelGGL(token_shift_mix_kernel<bf16s>, dim3(R), dim3(256), 0, s,
+                       (bf16s*)out, x, (const bf16s*)mu, state, tok_seq, seg_start,
+                       seg_len, seg_slot, seg_fresh, n_mix, R, W);
+}

@@ -31,7 +31,8 @@ CSRC = Path(__file__).resolve().parent / "csrc"
 SOURCES = [
     "group_norm.hip", "xielu.hip", "mingru.hip", "attention_general.hip",
     "attention_prefill_tiles.hip", "shift_norm.hip", "latent_attention.hip", "ff_act.hip",
-    "attention_latent_rows.hip",
+    "attention_latent_rows.hip", "post_norm.hip", "qkv_prep.hip", "attention_mixed_heads.hip",
+    "matrix_state_scan.hip",
 ]
 SO_PATH = PKG / "_hybrid.so"
 
@@ -79,7 +80,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "lig_sigmoid_gate_mul": [p, p, l, i, i, i, p],
         "lig_mingru_scan": [p, p, p, p, l, p, p, p, p, p, p, i, i, i, i, p],
         "lig_paged_attention_general": [
-            p, p, l, p, p, p, i, p, p, p, l, p, f, f, f, i, i, i, i, i, i, i, i, i, p,
+            p, p, l, p, p, p, i, p, p, p, l, p, f, f, f, i, i, i, i, i, i, i, i, i, i, p,
         ],
         "lig_offset_norm_shift": [p, p, p, p, p, p, p, p, p, p, p, p, p, p, p, f, i, i, i, p],
         "lig_offset_rms_norm": [p, p, p, f, i, i, i, p],
@@ -91,14 +92,29 @@ def _declare(lib: ctypes.CDLL) -> None:
         "lig_silu_mul": [p, p, l, i, i, p],
         "lig_kv_scatter": [p, p, l, p, p, p, i, i, i, i, i, i, p],
         "lig_temperature_scale_rows": [p, p, l, p, f, f, i, i, i, i, p],
+        "lig_scaled_add_rms_norm": [p, p, p, p, p, f, f, f, f, i, i, i, p],
+        "lig_qkv_norm_rope_cache": [
+            p, p, p, l, p, p, p, i, p, p, f, p, p, p, f, i, i, i, i, i, i, i, i, i, i, p,
+        ],
+        "lig_token_shift_mix": [p, p, p, p, p, p, p, p, p, i, i, i, i, p],
+        "lig_group_rms_norm_gate": [p, p, p, l, p, i, i, f, i, i, i, p],
+        "lig_gelu_erf": [p, p, l, i, p],
+        "lig_tanh_act": [p, p, l, i, p],
+        "lig_tanh_softcap": [p, f, l, p],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = None
     pt = lib.lig_paged_attention_prefill_tiles
-    pt.argtypes = [p, p, l, p, p, p, l, p, p, p, p, p, p, f, f, f, i, i, i, i, i, i, i, i, i, p]
+    pt.argtypes = [p, p, l, p, p, p, l, p, p, p, p, p, p, f, f, f, i, i, i, i, i, i, i, i, i, i, p]
     pt.restype = ctypes.c_int
+    mh = lib.lig_paged_attention_mixed_heads
+    mh.argtypes = [p, p, l, p, p, p, i, p, p, p, i, p, f, i, i, i, i, i, i, i, i, p]
+    mh.restype = ctypes.c_int
+    ms = lib.lig_matrix_state_scan
+    ms.argtypes = [p, p, l, p, l, p, l, p, p, p, p, l, p, p, p, p, i, i, i, i, i, i, p]
+    ms.restype = ctypes.c_int
     lr = lib.lig_latent_attention_rows
     lr.argtypes = [p, p, p, p, p, p, p, p, i, f, i, i, i, i, i, i, i, p, p]
     lr.restype = ctypes.c_int

@@ -291,13 +291,14 @@ def query_temperature(positions: torch.Tensor, coef: float, every: float) -> tor
 def paged_attention_general(
     q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float,
     num_heads: int, gate=None, temp_coef: float = 0.0, temp_every: float = 1.0,
-    sink=None,
+    sink=None, chunk: int = 0,
 ):
     """q [R, H*D] (may be a strided view); token r belongs to sequence row
     tok_seq[r] of block_tables (-1: padding row) and sees keys 0..positions[r].
     `sink` [H] fp32 adds exp(sink_h) to head h's softmax denominator (a key
     with that unscaled score and no value).  v_cache may be a view into
-    k_cache's rows."""
+    k_cache's rows.  chunk > 0 hides keys of earlier chunks: key j is seen
+    only if floor(j / chunk) == floor(position / chunk)."""
     R = q.shape[0]
     nb, G, bs, D = k_cache.shape
     Dv = v_cache.shape[-1]
@@ -328,6 +329,8 @@ def paged_attention_general(
             sc = torch.bmm(qf, kf.transpose(1, 2)) * (scale * tau[r:e])[None, :, None]
             keyp = torch.arange(L, device=q.device)[None, :]
             mask = keyp > positions[r:e, None]
+            if chunk > 0:
+                mask = mask | (keyp < (positions[r:e, None] // chunk) * chunk)
             sc.masked_fill_(mask[None], float("-inf"))
             if sink is not None:
                 sk = sink.float().view(H, 1, 1).expand(H, e - r, 1)
@@ -457,3 +460,184 @@ def scale_gather_rows(x, idx, w) -> torch.Tensor:
     ok = idx >= 0
     rows = x.float()[idx.clamp(min=0)] * (w.float() * ok)[:, None]
     return rows.to(x.dtype)
+
+
+# -- post-norm residual, query/key norms with rotation, chunked and head-mixed
+# -- attention, matrix-state recurrences ------------------------------------------
+
+def scaled_add_rms_norm(x, alpha: float, w, eps: float, y1=None, s1: float = 1.0,
+                        y2=None, s2: float = 1.0, out_dtype=None):
+    """Norm after the sum: x <- rms(alpha * x + s1 * y1 + s2 * y2) * w, x fp32
+    updated in place; also returned rounded to out_dtype.  Without y1 the
+    rows are only normed (x is left as it is)."""
+    if y1 is None:
+        return x, (_rms_scale(x, eps) * w.float()).to(out_dtype)
+    t = alpha * x + s1 * y1.float()
+    if y2 is not None:
+        t = t + s2 * y2.float()
+    x.copy_(_rms_scale(t, eps) * w.float())
+    return x, x.to(out_dtype)
+
+
+def _rotate_halves(v: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """v [R, heads, dim]: entry i pairs with entry i + n (n = len(inv_freq))
+    and the pair turns by positions * inv_freq[i]; entries from 2n on pass."""
+    n = inv_freq.shape[0]
+    out = v.float().clone()
+    ang = positions.float()[:, None] * inv_freq[None, :]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    a, b = out[..., :n].clone(), out[..., n : 2 * n].clone()
+    out[..., :n] = a * c - b * s
+    out[..., n : 2 * n] = b * c + a * s
+    return out
+
+
+def qkv_norm_rope_cache(
+    proj, heads: int, kv_heads: int, dim: int, vdim: int, qk_norm: str, w_q, w_k,
+    eps: float, inv_freq, positions, v_source: str, v_unit_norm: bool, v_first,
+    lam: float, want_v: bool, k_cache, v_cache, slot_mapping,
+):
+    R = proj.shape[0]
+    nq, nk = heads * dim, kv_heads * dim
+    q, k = proj[:, :nq].float(), proj[:, nq : nq + nk].float()
+    if v_source == "key":
+        v = k.clone().view(R, kv_heads, vdim)
+    else:
+        v = proj[:, nq + nk : nq + nk + kv_heads * vdim].float().reshape(R, kv_heads, vdim)
+    if qk_norm == "row":
+        q = (_rms_scale(q, eps) * w_q.float()).view(R, heads, dim)
+        k = (_rms_scale(k, eps) * w_k.float()).view(R, kv_heads, dim)
+    elif qk_norm == "head":
+        q = _rms_scale(q.reshape(R, heads, dim), eps) * w_q.float()
+        k = _rms_scale(k.reshape(R, kv_heads, dim), eps) * w_k.float()
+    else:
+        q, k = q.reshape(R, heads, dim), k.reshape(R, kv_heads, dim)
+    if inv_freq is not None and inv_freq.numel() > 0:
+        q = _rotate_halves(q, positions, inv_freq)
+        k = _rotate_halves(k, positions, inv_freq)
+    if v_unit_norm:
+        v = _rms_scale(v, eps)
+    if v_first is not None:
+        v = (1.0 - lam) * v + lam * v_first.view(R, kv_heads, vdim)
+    ok = slot_mapping >= 0
+    bs = k_cache.shape[2]
+    blk = torch.div(slot_mapping, bs, rounding_mode="floor")[ok]
+    off = (slot_mapping % bs)[ok]
+    k_cache[blk, :, off, :] = k[ok].to(k_cache.dtype)
+    v_cache[blk, :, off, :] = v[ok].to(v_cache.dtype)
+    return q.reshape(R, nq).to(proj.dtype), (v.reshape(R, kv_heads * vdim).clone() if want_v else None)
+
+
+def paged_attention_chunked(
+    q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float, num_heads: int,
+    chunk: int = 0, talk=None, dist_bias=None,
+):
+    """Token r sees keys j <= positions[r] of its sequence that lie in the
+    same chunk (floor(j / chunk) == floor(p / chunk); chunk 0: all of them).
+    Optional distance bias dist_bias[min(p - j, N - 1), head] added to the
+    scaled score, optional mixing of the heads' scores with talk [H, H]
+    before the softmax."""
+    R = q.shape[0]
+    nb, G, bs, D = k_cache.shape
+    Dv = v_cache.shape[-1]
+    H = num_heads
+    out = torch.zeros(R, H * Dv, dtype=q.dtype, device=q.device)
+    seqs, pos = tok_seq.tolist(), positions.tolist()
+    for r in range(R):
+        s, p = seqs[r], pos[r]
+        if s < 0:
+            continue
+        lo = (p // chunk) * chunk if chunk > 0 else 0
+        js = torch.arange(lo, p + 1, device=q.device)
+        blk = block_tables[s].long()[js // bs]
+        k = k_cache[blk, :, js % bs, :].float().repeat_interleave(H // G, dim=1)  # [L, H, D]
+        v = v_cache[blk, :, js % bs, :].float().repeat_interleave(H // G, dim=1)
+        sc = torch.einsum("hd,lhd->hl", q[r].float().view(H, D), k) * scale
+        if dist_bias is not None:
+            sc = sc + dist_bias.float()[(p - js).clamp(max=dist_bias.shape[0] - 1)].t()
+        if talk is not None:
+            sc = talk.float() @ sc
+        pr = torch.softmax(sc, dim=-1)
+        out[r] = torch.einsum("hl,lhd->hd", pr, v).reshape(H * Dv).to(out.dtype)
+    return out
+
+
+def token_shift_mix(x, mu, state, seg_start, seg_len, seg_slot, seg_fresh, out_dtype):
+    """out[m] = x + (x_prev - x) * mu[m] for every row of every segment; the
+    row before a segment's first is the sequence's state (zeros when the
+    sequence starts here), which then takes the segment's last row.  Rows of
+    no segment come out zero.  x fp32 [R, W], mu [n, W] -> [n, R, W]."""
+    prev = torch.zeros_like(x)
+    live = torch.zeros(x.shape[0], 1, dtype=torch.float32, device=x.device)
+    for s0, cnt, slot, fresh in zip(
+        seg_start.tolist(), seg_len.tolist(), seg_slot.tolist(), seg_fresh.tolist()
+    ):
+        if cnt <= 0:
+            continue
+        if not fresh:
+            prev[s0] = state[slot]
+        prev[s0 + 1 : s0 + cnt] = x[s0 : s0 + cnt - 1]
+        state[slot] = x[s0 + cnt - 1]
+        live[s0 : s0 + cnt] = 1.0
+    return ((x[None] + (prev - x)[None] * mu.float()[:, None, :]) * live[None]).to(out_dtype)
+
+
+def matrix_state_scan(
+    q, k, v, state, seg_start, seg_len, seg_slot, seg_fresh, heads: int, dim: int,
+    vdim: int, decay_pre=None, head_decay=None, bonus=None, act_silu: bool = False,
+):
+    """Per head a [dim, vdim] fp32 state S.  With `bonus` u (per head and key
+    channel): o_t = (S + diag(u) k_t v_t^T)^T q_t, then S <- diag(w_t) S +
+    k_t v_t^T with w_t = exp(-exp(decay_pre_t)).  Without: S <- d_h S + k_t
+    v_t^T with the head's constant d_h, then o_t = S^T q_t.  act_silu applies
+    silu to q, k and v first.  State rows [slots, heads*dim*vdim] are read
+    unless the segment starts its sequence, and written back."""
+    R = q.shape[0]
+    f = (lambda t: torch.nn.functional.silu(t.float())) if act_silu else (lambda t: t.float())
+    qf, kf, vf = f(q).view(R, heads, dim), f(k).view(R, heads, dim), f(v).view(R, heads, vdim)
+    out = torch.zeros(R, heads, vdim, dtype=torch.float32, device=q.device)
+    w = None
+    if decay_pre is not None:
+        w = torch.exp(-torch.exp(decay_pre.float())).view(R, heads, dim)
+    for s0, n, slot, fresh in zip(
+        seg_start.tolist(), seg_len.tolist(), seg_slot.tolist(), seg_fresh.tolist()
+    ):
+        if n <= 0:
+            continue
+        S = (
+            torch.zeros(heads, dim, vdim, dtype=torch.float32, device=q.device)
+            if fresh else state[slot, : heads * dim * vdim].view(heads, dim, vdim).clone()
+        )
+        for t in range(s0, s0 + n):
+            kv = kf[t][:, :, None] * vf[t][:, None, :]
+            if bonus is not None:
+                out[t] = torch.einsum("hd,hde->he", qf[t], S + bonus.float().view(heads, dim, 1) * kv)
+                S = w[t][:, :, None] * S + kv
+            else:
+                S = head_decay.float().view(heads, 1, 1) * S + kv
+                out[t] = torch.einsum("hd,hde->he", qf[t], S)
+        state[slot, : heads * dim * vdim] = S.reshape(-1)
+    return out.view(R, heads * vdim)
+
+
+def group_rms_norm_gate(o, gate, w, group: int, gate_act: str, eps: float, out_dtype):
+    """Every `group` consecutive entries of a row are divided by their root
+    mean square; then times w, times silu(gate) or sigmoid(gate)."""
+    R, C = o.shape
+    n = _rms_scale(o.view(R, C // group, group), eps).view(R, C) * w.float()
+    g = gate.float()
+    g = torch.nn.functional.silu(g) if gate_act == "silu" else torch.sigmoid(g)
+    return (n * g).to(out_dtype)
+
+
+def gelu_erf(x: torch.Tensor) -> torch.Tensor:
+    z = x.float()
+    return (0.5 * z * (1.0 + torch.erf(z * 0.7071067811865476))).to(x.dtype)
+
+
+def tanh_act(x: torch.Tensor) -> torch.Tensor:
+    return torch.tanh(x.float()).to(x.dtype)
+
+
+def tanh_softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    return x.copy_(cap * torch.tanh(x.float() / cap))
