@@ -74,6 +74,60 @@ def visibility(T: int, size: int):
     return np.array([[chunk_visible(i, j, size) for j in range(T)] for i in range(T)])
 
 
+def chunked_attention(q, k, v, scale: float, chunk: int, bias=None, talk=None):
+    """q [T, H, D], k [T, G, D], v [T, G, Dv] of one sequence -> [T, H, Dv].
+    Scores (q . k) * scale, plus bias [T, T, H] if given, then mixed across
+    heads with talk [H, H] if given; softmax over the keys of the query's
+    own chunk up to the query."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    s = np.zeros((H, T, T), F)
+    for hh in range(H):
+        s[hh] = q[:, hh] @ k[:, hh // (H // G)].T * scale
+        if bias is not None:
+            s[hh] += bias[:, :, hh]
+    if talk is not None:
+        s = np.einsum("hg,gij->hij", talk, s)
+    vis = visibility(T, chunk) if chunk > 0 else np.tril(np.ones((T, T), bool))
+    out = np.zeros((T, H, v.shape[2]), F)
+    for hh in range(H):
+        out[:, hh] = softmax_rows(s[hh], vis) @ v[:, hh // (H // G)]
+    return out
+
+
+def distance_bias(rel, T: int, far: float):
+    """bias[i, j, h] = rel[bucket(i - j), h] for j <= i."""
+    bias = np.zeros((T, T, rel.shape[1]), F)
+    for i in range(T):
+        for j in range(i + 1):
+            bias[i, j] = rel[distance_bucket(i - j, rel.shape[0], far)]
+    return bias
+
+
+def bonus_recurrence(r, k, v, w, u, S0=None):
+    """r, k, w [T, D], v [T, Dv], u [D] of one head: o_t = (S + diag(u) k_t
+    v_t^T)^T r_t, then S <- diag(w_t) S + k_t v_t^T.  Returns (o, S)."""
+    T, D = k.shape
+    S = np.zeros((D, v.shape[1]), F) if S0 is None else S0.copy()
+    o = np.zeros((T, v.shape[1]), F)
+    for i in range(T):
+        kv = np.outer(k[i], v[i])
+        o[i] = (S + u[:, None] * kv).T @ r[i]
+        S = w[i][:, None] * S + kv
+    return o, S
+
+
+def decay_recurrence(q, k, v, d: float, S0=None):
+    """S <- d S + k_t v_t^T, then o_t = S^T q_t.  Returns (o, S)."""
+    T, D = k.shape
+    S = np.zeros((D, v.shape[1]), F) if S0 is None else S0.copy()
+    o = np.zeros((T, v.shape[1]), F)
+    for i in range(T):
+        S = d * S + np.outer(k[i], v[i])
+        o[i] = S.T @ q[i]
+    return o, S
+
+
 def attention_mixer(h, t: Dict[str, np.ndarray], m: dict, eps: float, v_first: Optional[np.ndarray]):
     """Softmax attention with whole-projection query/key norms, partial
     rotate-half rotation, unit-RMS values, optional value mixing with the
@@ -96,12 +150,7 @@ def attention_mixer(h, t: Dict[str, np.ndarray], m: dict, eps: float, v_first: O
     if m.get("v_mix") and v_first is not None:
         lam = float(t["vmix"])
         v = (1.0 - lam) * v + lam * v_first
-    vis = visibility(T, m["mask"]["size"])
-    out = np.zeros((T, H, Dv), F)
-    for hh in range(H):
-        g = hh // (H // G)
-        p = softmax_rows(q[:, hh] @ k[:, g].T * m["scale"], vis)
-        out[:, hh] = p @ v[:, g]
+    out = chunked_attention(q, k, v, m["scale"], (m.get("mask") or {}).get("size", 0))
     return out.reshape(T, H * Dv) @ t["o"].T + t["o.b"], v
 
 
@@ -125,11 +174,7 @@ def wkv_mixer(h, t: Dict[str, np.ndarray], m: dict, eps: float):
     u = t["u"].reshape(H, D)
     o = np.zeros((T, H, D), F)
     for hh in range(H):
-        S = np.zeros((D, D), F)  # [key channel, value channel]
-        for i in range(T):
-            kv = np.outer(k[i, hh], v[i, hh])
-            o[i, hh] = (S + u[hh][:, None] * kv).T @ r[i, hh]
-            S = w[i, hh][:, None] * S + kv
+        o[:, hh], _ = bonus_recurrence(r[:, hh], k[:, hh], v[:, hh], w[:, hh], u[hh])
     o = rms(o, eps).reshape(T, H * D) * t["norm"] * gate
     return o @ t["o"].T
 
@@ -145,22 +190,10 @@ def shared_kv_attention(h, t: Dict[str, np.ndarray], m: dict, eps: float):
     v = k
     q = rms(q, eps) * t["q.norm"]
     k = rms(k, eps) * t["k.norm"]
-    rel = t["rel"]
-    rows = rel.shape[0]
-    bias = np.zeros((T, T, H), F)
-    for i in range(T):
-        for j in range(i + 1):
-            bias[i, j] = rel[distance_bucket(i - j, rows, m["bias_max"])]
-    s = np.zeros((H, T, T), F)
-    for hh in range(H):
-        g = hh // (H // G)
-        s[hh] = q[:, hh] @ k[:, g].T * m["scale"] + bias[:, :, hh]
-    s = np.einsum("hg,gij->hij", t["talk"], s)
-    vis = visibility(T, m["mask"]["size"])
-    out = np.zeros((T, H, D), F)
-    for hh in range(H):
-        g = hh // (H // G)
-        out[:, hh] = softmax_rows(s[hh], vis) @ v[:, g]
+    out = chunked_attention(
+        q, k, v, m["scale"], (m.get("mask") or {}).get("size", 0),
+        bias=distance_bias(t["rel"], T, m["bias_max"]), talk=t["talk"],
+    )
     return out.reshape(T, H * D) @ t["o"].T + t["o.b"]
 
 
@@ -173,10 +206,7 @@ def decay_mixer(h, t: Dict[str, np.ndarray], m: dict, eps: float):
     v = silu(h @ t["v"].T).reshape(T, H, Dv)
     o = np.zeros((T, H, Dv), F)
     for hh in range(H):
-        S = np.zeros((D, Dv), F)
-        for i in range(T):
-            S = m["decay"][hh] * S + np.outer(k[i, hh], v[i, hh])
-            o[i, hh] = S.T @ q[i, hh]
+        o[:, hh], _ = decay_recurrence(q[:, hh], k[:, hh], v[:, hh], m["decay"][hh])
     o = rms(o.reshape(T, H * Dv), eps) * t["norm"] * sigmoid(h @ t["g"].T)
     return o @ t["o"].T
 
