@@ -119,7 +119,27 @@ def main() -> None:
         "engine, kernels or both (benchmarks/bench_latent.py)",
     )
     ap.add_argument("--latent-sizes", default="s,m")
+    ap.add_argument(
+        "--postnorm",
+        nargs="?",
+        const="engine,kernels",
+        default="",
+        metavar="PARTS",
+        help="instead of the serving workload: Potatar (post-norm stack of "
+        "chunked attention, matrix-state recurrences and head-mixed "
+        "attention) beside Tikarax at equal size, and its kernels beside "
+        "their counterparts against the roofline; PARTS = engine, kernels or "
+        "both (benchmarks/bench_postnorm.py)",
+    )
+    ap.add_argument("--postnorm-sizes", default="s,m")
     args = ap.parse_args()
+
+    if args.postnorm:
+        sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmarks"))
+        import bench_postnorm
+
+        bench_postnorm.main(["--part", args.postnorm, "--sizes", args.postnorm_sizes])
+        return
 
     if args.latent:
         sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmarks"))

@@ -669,6 +669,12 @@ class MatrixStateMixer(nn.Module):
             self.norm.copy_(get(prefix + "norm"))
             self.w_o.copy_(get(prefix + "o"))
 
+    @staticmethod
+    def _zero_pad_rows(o, meta) -> None:
+        covered = meta.num_prefill_tokens + meta.num_decode_tokens
+        if covered < o.shape[0]:
+            o[covered:].zero_()  # GEMM-bucketing pad rows belong to no segment
+
     def forward(self, x, h, cache, meta, proj=None):
         """x: the fp32 rows (token shift reads them), h: the same in the
         activation dtype."""
@@ -683,6 +689,7 @@ class MatrixStateMixer(nn.Module):
                 rkvg[0], rkvg[1], rkvg[2], mat_state, *seg, self.heads, self.dim, self.vdim,
                 decay_pre=decay_pre, bonus=self.bonus,
             )
+            self._zero_pad_rows(o, meta)
             g = ops.group_rms_norm_gate(o, rkvg[3], self.norm, self.vdim, "silu", self.eps)
         else:
             (mat_state,) = cache
@@ -693,6 +700,7 @@ class MatrixStateMixer(nn.Module):
                 proj[:, :a], proj[:, a:b], proj[:, b:c], mat_state, *seg, self.heads,
                 self.dim, self.vdim, head_decay=self.head_decay, act_silu=True,
             )
+            self._zero_pad_rows(o, meta)
             g = ops.group_rms_norm_gate(o, proj[:, c : c + self.nv], self.norm, self.nv, "sigmoid", self.eps)
         return F.linear(g, self.w_o)
 

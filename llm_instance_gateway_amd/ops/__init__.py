@@ -1042,7 +1042,7 @@ def matrix_state_scan(
     act_silu applies silu to q, k, v on the way in.  state [slots,
     matrix_state_width] is read unless the segment starts its sequence and
     written back; its layout is private to the implementation.  Returns fp32
-    [R, heads*vdim]; rows of no segment are zero."""
+    [R, heads*vdim]; rows of no segment are left untouched (undefined)."""
     assert (bonus is None) == (decay_pre is None) and (bonus is None) != (head_decay is None)
     assert state.dtype == torch.float32
     if _use_hybrid(q):
@@ -1055,7 +1055,7 @@ def matrix_state_scan(
             if t is not None:
                 assert t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n
         S = seg_start.shape[0]
-        out = torch.zeros(R, heads * vdim, dtype=torch.float32, device=q.device)
+        out = torch.empty(R, heads * vdim, dtype=torch.float32, device=q.device)
         rc = _hl().lig_matrix_state_scan(
             _ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
             _ptr(decay_pre), _ptr(head_decay), _ptr(bonus), _ptr(state), state.stride(0),

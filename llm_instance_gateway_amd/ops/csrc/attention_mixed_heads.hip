@@ -22,7 +22,7 @@
 #define MH_MAX_HPW 4     // heads per wave: H <= 16 * 4
 #define MH_MAX_DVL 4     // value columns per lane: Dv <= 256
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ void paged_attention_mixed_heads_kernel(
     T* __restrict__ out, const T* __restrict__ q, long q_stride,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -84,7 +84,16 @@ __global__ void paged_attention_mixed_heads_kernel(
           const T* krow = k_cache + (kbase + (long)g * BS) * D;
           const float* qh = q_s + h * D;
           float dot = 0.f;
-          for (int d = 0; d < D; ++d) dot += qh[d] * ld(krow + d);
+          if (VEC) {  // D % 8 == 0 and 16-byte aligned rows
+            for (int d = 0; d < D; d += 8) {
+              float kv[8];
+              ld8(krow + d, kv);
+#pragma unroll
+              for (int i = 0; i < 8; ++i) dot += qh[d + i] * kv[i];
+            }
+          } else {
+            for (int d = 0; d < D; ++d) dot += qh[d] * ld(krow + d);
+          }
           a = dot * scale;
           if (dist_bias != nullptr) a += dist_bias[(long)min(pos - j, n_dist - 1) * H + h];
         }
@@ -151,17 +160,18 @@ extern "C" int lig_paged_attention_mixed_heads(
       (size_t)(H * D + 2 * H * WAVE_SIZE + ((H * H + 1) & ~1)) * sizeof(float) +
       WAVE_SIZE * sizeof(long);
   if (smem > 64 * 1024) return 1;
-  if (is_f32)
-    hipLaunchKernelGGL(paged_attention_mixed_heads_kernel<float>, dim3(R),
-                       dim3(nw * WAVE_SIZE), smem, s, (float*)out, (const float*)q,
-                       q_stride, (const float*)k_cache, (const float*)v_cache,
-                       block_tables, max_blocks, tok_seq, positions, dist_bias, n_dist,
-                       talk, scale, chunk, H, G, D, Dv, BS);
-  else
-    hipLaunchKernelGGL(paged_attention_mixed_heads_kernel<bf16s>, dim3(R),
-                       dim3(nw * WAVE_SIZE), smem, s, (bf16s*)out, (const bf16s*)q,
-                       q_stride, (const bf16s*)k_cache, (const bf16s*)v_cache,
-                       block_tables, max_blocks, tok_seq, positions, dist_bias, n_dist,
-                       talk, scale, chunk, H, G, D, Dv, BS);
+  const bool vec = D % 8 == 0 && aligned16(k_cache);
+#define LIG_MH(T, VEC)                                                              \
+  hipLaunchKernelGGL((paged_attention_mixed_heads_kernel<T, VEC>), dim3(R),         \
+                     dim3(nw * WAVE_SIZE), smem, s, (T*)out, (const T*)q, q_stride, \
+                     (const T*)k_cache, (const T*)v_cache, block_tables,            \
+                     max_blocks, tok_seq, positions, dist_bias, n_dist, talk,       \
+                     scale, chunk, H, G, D, Dv, BS)
+  if (is_f32) {
+    if (vec) LIG_MH(float, true); else LIG_MH(float, false);
+  } else {
+    if (vec) LIG_MH(bf16s, true); else LIG_MH(bf16s, false);
+  }
+#undef LIG_MH
   return 0;
 }

@@ -26,7 +26,9 @@
 
 #define MS_SPLIT 4
 
-template <typename T, int KMAX, bool BONUS>
+// EXACT: kpt == KMAX and a multiple of 4, so the per-token loop has constant
+// bounds and reads q, k and the decay from LDS four entries at a time.
+template <typename T, int KMAX, bool BONUS, bool EXACT>
 __global__ void matrix_state_scan_kernel(
     float* __restrict__ out,  // [R, H*Dv]
     const T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
@@ -103,16 +105,38 @@ __global__ void matrix_state_scan_kernel(
         const float* kt = k_s + t * Dp + s * kpt;
         const float* wt = w_s + t * Dp + s * kpt;
         float o = 0.f;
+        if (EXACT) {
 #pragma unroll
-        for (int ii = 0; ii < KMAX; ++ii) {
-          if (ii < kpt) {
-            const float kv = kt[ii] * vj;
-            if (BONUS) {
-              o += qt[ii] * (S[ii] + U[ii] * kv);
-              S[ii] = wt[ii] * S[ii] + kv;
-            } else {
-              S[ii] = dconst * S[ii] + kv;
-              o += qt[ii] * S[ii];
+          for (int i4 = 0; i4 < KMAX; i4 += 4) {
+            const f32x4 k4 = *reinterpret_cast<const f32x4*>(kt + i4);
+            const f32x4 q4 = *reinterpret_cast<const f32x4*>(qt + i4);
+            f32x4 w4 = {0.f, 0.f, 0.f, 0.f};
+            if (BONUS) w4 = *reinterpret_cast<const f32x4*>(wt + i4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int ii = i4 + e;
+              const float kv = k4[e] * vj;
+              if (BONUS) {
+                o += q4[e] * (S[ii] + U[ii] * kv);
+                S[ii] = w4[e] * S[ii] + kv;
+              } else {
+                S[ii] = dconst * S[ii] + kv;
+                o += q4[e] * S[ii];
+              }
+            }
+          }
+        } else {
+#pragma unroll
+          for (int ii = 0; ii < KMAX; ++ii) {
+            if (ii < kpt) {
+              const float kv = kt[ii] * vj;
+              if (BONUS) {
+                o += qt[ii] * (S[ii] + U[ii] * kv);
+                S[ii] = wt[ii] * S[ii] + kv;
+              } else {
+                S[ii] = dconst * S[ii] + kv;
+                o += qt[ii] * S[ii];
+              }
             }
           }
         }
@@ -146,18 +170,22 @@ extern "C" int lig_matrix_state_scan(
   const size_t smem = (size_t)per_tok * TT * sizeof(float);
   const int threads = ((Dv * MS_SPLIT + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE;
   dim3 grid(S, H), block(threads);
-#define LIG_MS(T, KMAX, B)                                                      \
-  hipLaunchKernelGGL((matrix_state_scan_kernel<T, KMAX, B>), grid, block, smem, \
-                     stream, out, (const T*)q, q_stride, (const T*)k, k_stride, \
-                     (const T*)v, v_stride, decay_pre, head_decay, bonus, state, \
-                     state_stride, seg_start, seg_len, seg_slot, seg_fresh, H,  \
-                     D, Dv, kpt, TT, act_silu)
+#define LIG_MS(T, KMAX, B, E)                                                   \
+  hipLaunchKernelGGL((matrix_state_scan_kernel<T, KMAX, B, E>), grid, block,    \
+                     smem, stream, out, (const T*)q, q_stride, (const T*)k,     \
+                     k_stride, (const T*)v, v_stride, decay_pre, head_decay,    \
+                     bonus, state, state_stride, seg_start, seg_len, seg_slot,  \
+                     seg_fresh, H, D, Dv, kpt, TT, act_silu)
 #define LIG_MS_K(T, B)                                    \
   do {                                                    \
-    if (kpt <= 8) LIG_MS(T, 8, B);                        \
-    else if (kpt <= 16) LIG_MS(T, 16, B);                 \
-    else if (kpt <= 32) LIG_MS(T, 32, B);                 \
-    else LIG_MS(T, 64, B);                                \
+    if (kpt == 8) LIG_MS(T, 8, B, true);                  \
+    else if (kpt < 8) LIG_MS(T, 8, B, false);             \
+    else if (kpt == 16) LIG_MS(T, 16, B, true);           \
+    else if (kpt < 16) LIG_MS(T, 16, B, false);           \
+    else if (kpt == 32) LIG_MS(T, 32, B, true);           \
+    else if (kpt < 32) LIG_MS(T, 32, B, false);           \
+    else if (kpt == 64) LIG_MS(T, 64, B, true);           \
+    else LIG_MS(T, 64, B, false);                         \
   } while (0)
   if (is_f32) {
     if (has_bonus) LIG_MS_K(float, true); else LIG_MS_K(float, false);

@@ -18,7 +18,9 @@
 
 #include "elem_types.h"
 
-template <typename T>
+// VEC: every block of the row (q, k, v) and every head is a multiple of 8
+// entries and 16-byte aligned, so global loads and stores move 8 at a time.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void qkv_norm_rope_cache_kernel(
     T* __restrict__ q_out, float* __restrict__ v_out, const T* __restrict__ proj,
     long proj_stride, const T* __restrict__ w_q, const T* __restrict__ w_k,
@@ -38,14 +40,25 @@ __global__ __launch_bounds__(256) void qkv_norm_rope_cache_kernel(
   const int tid = threadIdx.x, nt = blockDim.x;
   const int wave = tid / WAVE_SIZE, lane = tid % WAVE_SIZE, nwaves = nt / WAVE_SIZE;
 
-  for (int c = tid; c < nq; c += nt) q_s[c] = ld(row + c);
-  for (int c = tid; c < nk; c += nt) {
-    const float kv = ld(row + nq + c);
-    k_s[c] = kv;
-    if (v_from_key) v_s[c] = kv;  // Dv == D
+  if (VEC) {
+    // q_s, k_s, v_s are contiguous in LDS just as q | k | v are in the row
+    const int n_in = nq + nk + (v_from_key ? 0 : nv);
+    for (int c = tid * 8; c < n_in; c += nt * 8) {
+      float t[8];
+      ld8(row + c, t);
+      st8(sm + c, t);
+      if (v_from_key && c >= nq) st8(v_s + (c - nq), t);  // Dv == D
+    }
+  } else {
+    for (int c = tid; c < nq; c += nt) q_s[c] = ld(row + c);
+    for (int c = tid; c < nk; c += nt) {
+      const float kv = ld(row + nq + c);
+      k_s[c] = kv;
+      if (v_from_key) v_s[c] = kv;  // Dv == D
+    }
+    if (!v_from_key)
+      for (int c = tid; c < nv; c += nt) v_s[c] = ld(row + nq + nk + c);
   }
-  if (!v_from_key)
-    for (int c = tid; c < nv; c += nt) v_s[c] = ld(row + nq + nk + c);
   __syncthreads();
 
   if (norm_mode == 1) {
@@ -104,13 +117,36 @@ __global__ __launch_bounds__(256) void qkv_norm_rope_cache_kernel(
     __syncthreads();
   }
 
-  for (int c = tid; c < nq; c += nt) st(q_out + r * nq + c, q_s[c]);
+  if (VEC) {
+    for (int c = tid * 8; c < nq; c += nt * 8) {
+      float t[8];
+      ld8(q_s + c, t);
+      st8(q_out + r * nq + c, t);
+    }
+  } else {
+    for (int c = tid; c < nq; c += nt) st(q_out + r * nq + c, q_s[c]);
+  }
   if (v_out != nullptr)
     for (int c = tid; c < nv; c += nt) v_out[r * nv + c] = v_s[c];
   const int64_t slot = slot_mapping[r];
   if (slot < 0) return;
   const long blk = slot / BS;
   const int off = (int)(slot % BS);
+  if (VEC) {
+    for (int c = tid * 8; c < nk + nv; c += nt * 8) {
+      float t[8];
+      if (c < nk) {
+        const int g = c / D, d = c - g * D;
+        ld8(k_s + c, t);
+        st8(k_cache + ((blk * G + g) * BS + off) * (long)D + d, t);
+      } else {
+        const int e = c - nk, g = e / Dv, d = e - g * Dv;
+        ld8(v_s + e, t);
+        st8(v_cache + ((blk * G + g) * BS + off) * (long)Dv + d, t);
+      }
+    }
+    return;
+  }
   for (int c = tid; c < nk; c += nt) {
     const int g = c / D, d = c - g * D;
     st(k_cache + ((blk * G + g) * BS + off) * (long)D + d, k_s[c]);
@@ -130,18 +166,18 @@ extern "C" void lig_qkv_norm_rope_cache(
     hipStream_t s) {
   if (R <= 0) return;
   const size_t smem = (size_t)(H * D + G * D + G * Dv) * sizeof(float);
-  if (is_f32)
-    hipLaunchKernelGGL(qkv_norm_rope_cache_kernel<float>, dim3(R), dim3(256), smem, s,
-                       (float*)q_out, v_out, (const float*)proj, proj_stride,
-                       (const float*)w_q, (const float*)w_k, inv_freq, n_freq,
-                       positions, v_first, lam, (float*)k_cache, (float*)v_cache,
-                       slot_mapping, eps, H, G, D, Dv, norm_mode, v_from_key,
-                       v_unit_norm, BS);
-  else
-    hipLaunchKernelGGL(qkv_norm_rope_cache_kernel<bf16s>, dim3(R), dim3(256), smem, s,
-                       (bf16s*)q_out, v_out, (const bf16s*)proj, proj_stride,
-                       (const bf16s*)w_q, (const bf16s*)w_k, inv_freq, n_freq,
-                       positions, v_first, lam, (bf16s*)k_cache, (bf16s*)v_cache,
-                       slot_mapping, eps, H, G, D, Dv, norm_mode, v_from_key,
-                       v_unit_norm, BS);
+  const bool vec = D % 8 == 0 && Dv % 8 == 0 && proj_stride % 8 == 0 && aligned16(proj) &&
+                   aligned16(q_out) && aligned16(k_cache) && aligned16(v_cache);
+#define LIG_QP(T, VEC)                                                              \
+  hipLaunchKernelGGL((qkv_norm_rope_cache_kernel<T, VEC>), dim3(R), dim3(256), smem, \
+                     s, (T*)q_out, v_out, (const T*)proj, proj_stride,              \
+                     (const T*)w_q, (const T*)w_k, inv_freq, n_freq, positions,     \
+                     v_first, lam, (T*)k_cache, (T*)v_cache, slot_mapping, eps, H,  \
+                     G, D, Dv, norm_mode, v_from_key, v_unit_norm, BS)
+  if (is_f32) {
+    if (vec) LIG_QP(float, true); else LIG_QP(float, false);
+  } else {
+    if (vec) LIG_QP(bf16s, true); else LIG_QP(bf16s, false);
+  }
+#undef LIG_QP
 }

@@ -394,6 +394,56 @@ __global__ __launch_bounds__(256) void token_shift_mix_kernel(
   }
 }
 
+// 8 elements per thread and access: W % 8 == 0, 16-byte aligned rows.
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_mix_vec_kernel(
+    T* __restrict__ out, const float* __restrict__ x, const T* __restrict__ mu,
+    float* __restrict__ state, const int* __restrict__ tok_seq,
+    const int* __restrict__ seg_start, const int* __restrict__ seg_len,
+    const int* __restrict__ seg_slot, const int* __restrict__ seg_fresh,
+    int n_mix, int R, int W) {
+  const long r = blockIdx.x;
+  const int seq = tok_seq[r];
+  if (seq < 0) {
+    float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int m = 0; m < n_mix; ++m)
+      for (int c = threadIdx.x * 8; c < W; c += blockDim.x * 8)
+        st8(out + ((long)m * R + r) * W + c, z);
+    return;
+  }
+  const int s0 = seg_start[seq];
+  const bool first = r == s0;
+  const float* prev = nullptr;
+  float* srow = state + (long)seg_slot[seq] * W;
+  if (!first) prev = x + (r - 1) * W;
+  else if (!seg_fresh[seq]) prev = srow;
+  const float* last = x + ((long)s0 + seg_len[seq] - 1) * W;
+  for (int c = threadIdx.x * 8; c < W; c += blockDim.x * 8) {
+    float cur[8], d[8];
+    ld8(x + r * W + c, cur);
+    if (prev != nullptr) {
+      ld8(prev + c, d);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) d[i] -= cur[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) d[i] = -cur[i];
+    }
+    for (int m = 0; m < n_mix; ++m) {
+      float u[8];
+      ld8(mu + (long)m * W + c, u);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) u[i] = cur[i] + d[i] * u[i];
+      st8(out + ((long)m * R + r) * W + c, u);
+    }
+    if (first) {  // after this thread's own read of srow[c..c+8)
+      float l8[8];
+      ld8(last + c, l8);
+      st8(srow + c, l8);
+    }
+  }
+}
+
 extern "C" void lig_token_shift_mix(void* out, const float* x, const void* mu,
                                     float* state, const int* tok_seq,
                                     const int* seg_start, const int* seg_len,
@@ -401,6 +451,17 @@ extern "C" void lig_token_shift_mix(void* out, const float* x, const void* mu,
                                     int n_mix, int R, int W, int is_f32,
                                     hipStream_t s) {
   if (R <= 0 || W <= 0) return;
+  if (W % 8 == 0 && aligned16(out) && aligned16(x) && aligned16(mu) && aligned16(state)) {
+    if (is_f32)
+      hipLaunchKernelGGL(token_shift_mix_vec_kernel<float>, dim3(R), dim3(256), 0, s,
+                         (float*)out, x, (const float*)mu, state, tok_seq, seg_start,
+                         seg_len, seg_slot, seg_fresh, n_mix, R, W);
+    else
+      hipLaunchKernelGGL(token_shift_mix_vec_kernel<bf16s>, dim3(R), dim3(256), 0, s,
+                         (bf16s*)out, x, (const bf16s*)mu, state, tok_seq, seg_start,
+                         seg_len, seg_slot, seg_fresh, n_mix, R, W);
+    return;
+  }
   if (is_f32)
     hipLaunchKernelGGL(token_shift_mix_kernel<float>, dim3(R), dim3(256), 0, s,
                        (float*)out, x, (const float*)mu, state, tok_seq, seg_start,
