@@ -1016,14 +1016,20 @@ def token_shift_mix(x, mu, state, tok_seq, seg_start, seg_len, seg_slot, seg_fre
 
 
 MATRIX_STATE_KEY_SPLIT = 4
+# key channels per thread the scan kernel is instantiated for
+MATRIX_STATE_KEY_CLASSES = (4, 8, 12, 16, 24, 32, 48, 64)
 
 
 def matrix_state_width(heads: int, dim: int, vdim: int) -> int:
     """fp32 entries of one sequence's matrix state: the scan kernel splits a
     head's key channels over four lanes and keeps the state in the order its
-    threads hold it, key channels padded to a multiple of four."""
-    k = MATRIX_STATE_KEY_SPLIT
-    return heads * ((dim + k - 1) // k) * k * vdim
+    threads hold it, key channels padded to four times the kernel's size
+    class."""
+    need = (dim + MATRIX_STATE_KEY_SPLIT - 1) // MATRIX_STATE_KEY_SPLIT
+    kpt = next((c for c in MATRIX_STATE_KEY_CLASSES if c >= need), None)
+    if kpt is None:
+        raise ValueError(f"matrix-state heads hold at most 256 key channels, got {dim}")
+    return heads * MATRIX_STATE_KEY_SPLIT * kpt * vdim
 
 
 def matrix_state_scan(

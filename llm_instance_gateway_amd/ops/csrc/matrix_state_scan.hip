@@ -10,7 +10,8 @@
 //   optional silu on q, k, v as they are read.
 //
 // One workgroup per (segment, head).  A thread owns value column j and one
-// quarter of the key channels (lane = 4 j + s, keys s*KPT .. s*KPT + KPT-1),
+// quarter of the key channels (lane = 4 j + s, keys s*KPT .. s*KPT + KPT-1,
+// KPT one of a few size classes),
 // keeps its KPT state entries in registers for the whole segment, and the
 // four partial outputs of a column are summed with two lane shuffles.  The
 // segment is walked serially, TT tokens staged into LDS at a time (q, k, the
@@ -19,17 +20,20 @@
 // depend on how a sequence is cut into steps.
 //
 // The state row of a sequence is stored in the order the threads hold it,
-// [head][ii][thread] with D padded to 4*KPT: loads and stores are coalesced.
+// [head][ii][thread] with D padded to 4*KPT: loads and stores are coalesced
+// (a row holds H * 4 * KPT * Dv entries; ops.matrix_state_width mirrors this).
 // A segment that starts its sequence ignores what the slot held.
 
 #include "elem_types.h"
 
 #define MS_SPLIT 4
 
-// EXACT: kpt == KMAX and a multiple of 4, so the per-token loop has constant
-// bounds and reads q, k and the decay from LDS four entries at a time.
-template <typename T, int KMAX, bool BONUS, bool EXACT>
-__global__ void matrix_state_scan_kernel(
+// KPT: key channels per thread (D is padded to 4 * KPT; padded channels carry
+// q = k = w = 0 and stay zero).  MAXT bounds the workgroup size (4 * Dv
+// rounded up to whole waves) so the compiler may use the register file a
+// small workgroup leaves it.
+template <typename T, int KPT, bool BONUS, int MAXT>
+__global__ __launch_bounds__(MAXT) void matrix_state_scan_kernel(
     float* __restrict__ out,  // [R, H*Dv]
     const T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
     const T* __restrict__ v, long v_stride,
@@ -38,10 +42,9 @@ __global__ void matrix_state_scan_kernel(
     const float* __restrict__ bonus,       // [H*D]      (BONUS)
     float* __restrict__ state, long state_stride, const int* __restrict__ seg_start,
     const int* __restrict__ seg_len, const int* __restrict__ seg_slot,
-    const int* __restrict__ seg_fresh, int H, int D, int Dv, int kpt, int TT,
-    int act_silu) {
+    const int* __restrict__ seg_fresh, int H, int D, int Dv, int TT, int act_silu) {
   extern __shared__ __align__(16) float sm[];
-  const int Dp = MS_SPLIT * kpt;
+  constexpr int Dp = MS_SPLIT * KPT;
   float* q_s = sm;                 // [TT][Dp]
   float* k_s = q_s + TT * Dp;      // [TT][Dp]
   float* w_s = k_s + TT * Dp;      // [TT][Dp] (BONUS only)
@@ -56,24 +59,22 @@ __global__ void matrix_state_scan_kernel(
   const bool owner = j < Dv;
   const int nthr = Dv * MS_SPLIT;  // threads that own state
 
-  float S[KMAX], U[KMAX];
-  float* srow = state + (long)seg_slot[seg] * state_stride + (long)h * kpt * nthr;
-  const bool fresh = seg_fresh[seg] != 0;
+  float S[KPT], U[KPT];
+  float* srow = state + (long)seg_slot[seg] * state_stride + (long)h * KPT * nthr;
+  const bool load_state = owner && seg_fresh[seg] == 0;
 #pragma unroll
-  for (int ii = 0; ii < KMAX; ++ii) {
-    S[ii] = 0.f;
-    U[ii] = 0.f;
-    if (ii < kpt && owner) {
-      if (!fresh) S[ii] = srow[(long)ii * nthr + tid];
-      const int i = s * kpt + ii;
-      if (BONUS && i < D) U[ii] = bonus[h * D + i];
-    }
+  for (int ii = 0; ii < KPT; ++ii) {
+    S[ii] = load_state ? srow[(long)ii * nthr + tid] : 0.f;
+    const int i = s * KPT + ii;
+    U[ii] = (BONUS && i < D) ? bonus[h * D + i] : 0.f;
   }
   const float dconst = BONUS ? 0.f : head_decay[h];
 
+#pragma nounroll
   for (int t0 = 0; t0 < n; t0 += TT) {
     const int nt_tok = min(TT, n - t0);
     __syncthreads();  // the previous tile's readers are done
+#pragma nounroll
     for (int e = tid; e < nt_tok * Dp; e += nt) {
       const int t = e / Dp, i = e - t * Dp;
       const long r = r0 + t0 + t;
@@ -91,6 +92,7 @@ __global__ void matrix_state_scan_kernel(
       k_s[e] = kv;
       if (BONUS) w_s[e] = wv;
     }
+#pragma nounroll
     for (int e = tid; e < nt_tok * Dv; e += nt) {
       const int t = e / Dv, c = e - t * Dv;
       float vv = ld(v + (long)(r0 + t0 + t) * v_stride + h * Dv + c);
@@ -98,59 +100,53 @@ __global__ void matrix_state_scan_kernel(
       v_s[e] = vv;
     }
     __syncthreads();
-    if (tid < ((nthr + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE) {  // whole waves: shuffles below
-      for (int t = 0; t < nt_tok; ++t) {
-        const float vj = owner ? v_s[t * Dv + j] : 0.f;
-        const float* qt = q_s + t * Dp + s * kpt;
-        const float* kt = k_s + t * Dp + s * kpt;
-        const float* wt = w_s + t * Dp + s * kpt;
-        float o = 0.f;
-        if (EXACT) {
+    // every wave of the workgroup walks the tile (idle lanes of the last
+    // wave take part in the shuffles with zeros)
+#pragma nounroll
+    for (int t = 0; t < nt_tok; ++t) {
+      const float vj = owner ? v_s[t * Dv + j] : 0.f;
+      const float* qt = q_s + t * Dp + s * KPT;
+      const float* kt = k_s + t * Dp + s * KPT;
+      const float* wt = w_s + t * Dp + s * KPT;
+      float o = 0.f;
 #pragma unroll
-          for (int i4 = 0; i4 < KMAX; i4 += 4) {
-            const f32x4 k4 = *reinterpret_cast<const f32x4*>(kt + i4);
-            const f32x4 q4 = *reinterpret_cast<const f32x4*>(qt + i4);
-            f32x4 w4 = {0.f, 0.f, 0.f, 0.f};
-            if (BONUS) w4 = *reinterpret_cast<const f32x4*>(wt + i4);
+      for (int i4 = 0; i4 < KPT; i4 += 4) {
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(kt + i4);
+        const f32x4 q4 = *reinterpret_cast<const f32x4*>(qt + i4);
+        f32x4 w4 = {0.f, 0.f, 0.f, 0.f};
+        if (BONUS) w4 = *reinterpret_cast<const f32x4*>(wt + i4);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int ii = i4 + e;
-              const float kv = k4[e] * vj;
-              if (BONUS) {
-                o += q4[e] * (S[ii] + U[ii] * kv);
-                S[ii] = w4[e] * S[ii] + kv;
-              } else {
-                S[ii] = dconst * S[ii] + kv;
-                o += q4[e] * S[ii];
-              }
-            }
-          }
-        } else {
-#pragma unroll
-          for (int ii = 0; ii < KMAX; ++ii) {
-            if (ii < kpt) {
-              const float kv = kt[ii] * vj;
-              if (BONUS) {
-                o += qt[ii] * (S[ii] + U[ii] * kv);
-                S[ii] = wt[ii] * S[ii] + kv;
-              } else {
-                S[ii] = dconst * S[ii] + kv;
-                o += qt[ii] * S[ii];
-              }
-            }
+        for (int e = 0; e < 4; ++e) {
+          const int ii = i4 + e;
+          const float kv = k4[e] * vj;
+          if (BONUS) {
+            o += q4[e] * (S[ii] + U[ii] * kv);
+            S[ii] = w4[e] * S[ii] + kv;
+          } else {
+            S[ii] = dconst * S[ii] + kv;
+            o += q4[e] * S[ii];
           }
         }
-        o += __shfl_xor(o, 1, WAVE_SIZE);
-        o += __shfl_xor(o, 2, WAVE_SIZE);
-        if (owner && s == 0) out[(long)(r0 + t0 + t) * (H * Dv) + h * Dv + j] = o;
       }
+      o += __shfl_xor(o, 1, WAVE_SIZE);
+      o += __shfl_xor(o, 2, WAVE_SIZE);
+      if (owner && s == 0) out[(long)(r0 + t0 + t) * (H * Dv) + h * Dv + j] = o;
     }
   }
   if (owner) {
 #pragma unroll
-    for (int ii = 0; ii < KMAX; ++ii)
-      if (ii < kpt) srow[(long)ii * nthr + tid] = S[ii];
+    for (int ii = 0; ii < KPT; ++ii) srow[(long)ii * nthr + tid] = S[ii];
   }
+}
+
+// Key channels per thread for a head of D key channels: the smallest size
+// class that holds ceil(D / 4); 0 when D is too wide.
+static int ms_keys_per_thread(int D) {
+  static const int classes[] = {4, 8, 12, 16, 24, 32, 48, 64};
+  const int need = (D + MS_SPLIT - 1) / MS_SPLIT;
+  for (int c : classes)
+    if (c >= need) return c;
+  return 0;
 }
 
 // Returns 0 when launched, 1 when a head is wider than the kernel holds.
@@ -160,9 +156,9 @@ extern "C" int lig_matrix_state_scan(
     const float* bonus, float* state, long state_stride, const int* seg_start,
     const int* seg_len, const int* seg_slot, const int* seg_fresh, int S, int H,
     int D, int Dv, int act_silu, int is_f32, hipStream_t stream) {
-  if (D <= 0 || Dv <= 0 || D > 256 || Dv > 256) return 1;
+  const int kpt = D > 0 ? ms_keys_per_thread(D) : 0;
+  if (kpt == 0 || Dv <= 0 || Dv > 256) return 1;
   if (S <= 0) return 0;
-  const int kpt = (D + MS_SPLIT - 1) / MS_SPLIT;
   const int Dp = kpt * MS_SPLIT;
   const bool has_bonus = bonus != nullptr;
   const int per_tok = (has_bonus ? 3 : 2) * Dp + Dv;
@@ -170,29 +166,35 @@ extern "C" int lig_matrix_state_scan(
   const size_t smem = (size_t)per_tok * TT * sizeof(float);
   const int threads = ((Dv * MS_SPLIT + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE;
   dim3 grid(S, H), block(threads);
-#define LIG_MS(T, KMAX, B, E)                                                   \
-  hipLaunchKernelGGL((matrix_state_scan_kernel<T, KMAX, B, E>), grid, block,    \
+#define LIG_MS_T(T, KPT, B, MAXT)                                               \
+  hipLaunchKernelGGL((matrix_state_scan_kernel<T, KPT, B, MAXT>), grid, block,  \
                      smem, stream, out, (const T*)q, q_stride, (const T*)k,     \
                      k_stride, (const T*)v, v_stride, decay_pre, head_decay,    \
                      bonus, state, state_stride, seg_start, seg_len, seg_slot,  \
-                     seg_fresh, H, D, Dv, kpt, TT, act_silu)
-#define LIG_MS_K(T, B)                                    \
-  do {                                                    \
-    if (kpt == 8) LIG_MS(T, 8, B, true);                  \
-    else if (kpt < 8) LIG_MS(T, 8, B, false);             \
-    else if (kpt == 16) LIG_MS(T, 16, B, true);           \
-    else if (kpt < 16) LIG_MS(T, 16, B, false);           \
-    else if (kpt == 32) LIG_MS(T, 32, B, true);           \
-    else if (kpt < 32) LIG_MS(T, 32, B, false);           \
-    else if (kpt == 64) LIG_MS(T, 64, B, true);           \
-    else LIG_MS(T, 64, B, false);                         \
+                     seg_fresh, H, D, Dv, TT, act_silu)
+#define LIG_MS(T, KPT, B)                               \
+  do {                                                  \
+    if (threads <= 256) LIG_MS_T(T, KPT, B, 256);       \
+    else LIG_MS_T(T, KPT, B, 1024);                     \
   } while (0)
+#define LIG_MS_K(T, B)                          \
+  switch (kpt) {                                \
+    case 4: LIG_MS(T, 4, B); break;             \
+    case 8: LIG_MS(T, 8, B); break;             \
+    case 12: LIG_MS(T, 12, B); break;           \
+    case 16: LIG_MS(T, 16, B); break;           \
+    case 24: LIG_MS(T, 24, B); break;           \
+    case 32: LIG_MS(T, 32, B); break;           \
+    case 48: LIG_MS(T, 48, B); break;           \
+    default: LIG_MS(T, 64, B); break;           \
+  }
   if (is_f32) {
-    if (has_bonus) LIG_MS_K(float, true); else LIG_MS_K(float, false);
+    if (has_bonus) { LIG_MS_K(float, true) } else { LIG_MS_K(float, false) }
   } else {
-    if (has_bonus) LIG_MS_K(bf16s, true); else LIG_MS_K(bf16s, false);
+    if (has_bonus) { LIG_MS_K(bf16s, true) } else { LIG_MS_K(bf16s, false) }
   }
 #undef LIG_MS_K
 #undef LIG_MS
+#undef LIG_MS_T
   return 0;
 }
