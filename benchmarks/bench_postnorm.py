@@ -207,6 +207,11 @@ def part_kernels(sizes) -> None:
                 vc2 = torch.randn_like(kc2)
                 q2 = torch.randn(T, lh * lD, device=dev, dtype=bf)
                 fl2 = 4.0 * Sq * pairs(CHUNK) * lD * lh
+                if ops.mixed_heads_tiles_supported(bf, lD, lD, lh, True):
+                    addf("paged_attention_mixed_heads_tiles(MFMA, bias + head mixing, chunked)", "paged_attention_prefill_tiles",
+                         timeit(lambda: ops.paged_attention_mixed_heads_tiles(
+                             q2, kc2, vc2, tables, qsl, ctxl, tseq, tqs, sc, lh, dist_bias=tab, talk=talk,
+                             chunk=CHUNK), 10), fl2)
                 addf("paged_attention_mixed_heads(bias + head mixing, chunked, prompt rows)", "",
                      timeit(lambda: ops.paged_attention_mixed_heads(
                          q2, kc2, vc2, tables, tsq, posq, sc, lh, dist_bias=tab, talk=talk, chunk=CHUNK), 3), fl2)

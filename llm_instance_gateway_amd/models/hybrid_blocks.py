@@ -551,15 +551,45 @@ class NormedRotaryAttention(nn.Module):
             v_first=v_first, lam=self.lam, want_v=want_v,
         )
         if self.mixes_heads:
-            o = ops.paged_attention_mixed_heads(
-                q, k_cache, v_cache, meta.seq_block_tables, meta.tok_seq, positions,
-                self.scale, self.heads, dist_bias=self.dist_bias, talk=self.talk,
-                chunk=self.chunk,
-            )
+            o = self._attend_mixed(q, positions, k_cache, v_cache, meta)
         else:
             o = self._attend(q, positions, k_cache, v_cache, meta)
         y = F.linear(o, self.w_o, self.b_o if self.has_bias else None)
         return (y, v_out) if want_v else y
+
+    def _attend_mixed(self, q, positions, k_cache, v_cache, meta):
+        """All heads of a token together: prompt portions on MFMA tiles where
+        the shape allows, everything else (single tokens, pad rows, fp32)
+        through the any-shape head-mixing kernel."""
+        np_, rows = meta.num_prefill_tokens, q.shape[0]
+        kw = dict(dist_bias=self.dist_bias, talk=self.talk, chunk=self.chunk)
+        done = 0
+        o = None
+        if (
+            np_ > 0
+            and meta.prefill_tile_seq is not None
+            and ops.mixed_heads_tiles_supported(q.dtype, self.dim, self.vdim, self.heads, q.is_cuda)
+        ):
+            o = torch.empty(rows, self.heads * self.vdim, dtype=q.dtype, device=q.device)
+            res = ops.paged_attention_mixed_heads_tiles(
+                q[:np_], k_cache, v_cache, meta.prefill_block_tables,
+                meta.prefill_query_start_locs, meta.prefill_context_lens,
+                meta.prefill_tile_seq, meta.prefill_tile_qstart, self.scale, self.heads,
+                out=o[:np_], **kw,
+            )
+            done = np_ if res is not None else 0
+        if done == rows:
+            return o
+        if done == 0:
+            return ops.paged_attention_mixed_heads(
+                q, k_cache, v_cache, meta.seq_block_tables, meta.tok_seq, positions,
+                self.scale, self.heads, **kw,
+            )
+        ops.paged_attention_mixed_heads(
+            q[done:], k_cache, v_cache, meta.seq_block_tables, meta.tok_seq[done:],
+            positions[done:], self.scale, self.heads, out=o[done:], **kw,
+        )
+        return o
 
     def _attend(self, q, positions, k_cache, v_cache, meta):
         np_, rows = meta.num_prefill_tokens, q.shape[0]

@@ -195,12 +195,22 @@ class PotatarForCausalLM(nn.Module):
         # ones blend in
         self.v_source = next((i for i, l in enumerate(self.layers) if l.v_mix), -1)
         self.v_users = sum(1 for l in self.layers if l.v_mix)
-        # prompt rows of plain attention layers run the MFMA tile kernel
-        # where the head sizes allow: the runner then builds 64-row tiles
+        # prompt rows of the attention layers (plain and head-mixed) run MFMA
+        # tile kernels where the shapes allow: the runner then builds 64-row
+        # tiles
         on_gpu = self.device_.type == "cuda"
         self.needs_prefill_tiles = any(
-            s.type == "attention"
-            and ops.tiled_prefill_supported(dtype, s.mixer["dim"], s.mixer["vdim"], on_gpu)
+            (
+                s.type == "attention"
+                and ops.tiled_prefill_supported(dtype, s.mixer["dim"], s.mixer["vdim"], on_gpu)
+            )
+            or (
+                s.type == "parallel"
+                and ops.mixed_heads_tiles_supported(
+                    dtype, s.mixer["left"]["dim"], s.mixer["left"]["dim"],
+                    s.mixer["left"]["heads"], on_gpu,
+                )
+            )
             for s in cfg.layer_specs
         )
         # test/debug hook: when a list, forward() appends the fp32 residual

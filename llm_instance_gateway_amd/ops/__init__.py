@@ -994,6 +994,58 @@ def paged_attention_mixed_heads(
     return res
 
 
+def mixed_heads_tiles_supported(q_dtype, k_dim: int, v_dim: int, heads: int, is_cuda: bool) -> bool:
+    """The MFMA head-mixing kernel for prompt rows: bf16, head sizes multiples
+    of 8 up to 128, at most 16 heads (one wave per head in a workgroup)."""
+    return (
+        is_cuda
+        and q_dtype == torch.bfloat16
+        and k_dim % 8 == 0
+        and v_dim % 8 == 0
+        and 0 < k_dim <= 128
+        and 0 < v_dim <= 128
+        and 1 <= heads <= 16
+        and os.environ.get("LIG_FORCE_TORCH_OPS") != "1"
+        and os.environ.get("LIG_GENERAL_ATTENTION") != "1"
+    )
+
+
+def paged_attention_mixed_heads_tiles(
+    q, k_cache, v_cache, block_tables, query_start_locs, context_lens, tile_seq,
+    tile_qstart, scale: float, num_heads: int, dist_bias: Optional[torch.Tensor] = None,
+    talk: Optional[torch.Tensor] = None, chunk: int = 0, out: Optional[torch.Tensor] = None,
+) -> Optional[torch.Tensor]:
+    """`paged_attention_mixed_heads` for the step's prompt portions on MFMA
+    tiles: q [Tp, H*D] (strided view allowed) laid out by query_start_locs,
+    context_lens count each sequence's tokens after this step, tile_seq /
+    tile_qstart name the 64-row query tiles (each is run as four 16-row
+    workgroups that hold all heads).  Returns None when the shape does not
+    fit the kernel's LDS budget (the caller then uses the any-shape kernel).
+    GPU, bf16."""
+    nb, G, bs, D = k_cache.shape
+    Dv = v_cache.shape[-1]
+    Tp = q.shape[0]
+    assert q.is_cuda and q.dtype == torch.bfloat16 and q.stride(1) == 1
+    assert q.shape[1] == num_heads * D and k_cache.is_contiguous() and v_cache.is_contiguous()
+    for t in (block_tables, query_start_locs, context_lens, tile_seq, tile_qstart):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    for t in (dist_bias, talk):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous())
+    assert dist_bias is None or (dist_bias.dim() == 2 and dist_bias.shape[1] == num_heads)
+    assert talk is None or talk.shape == (num_heads, num_heads)
+    if out is None:
+        out = torch.empty(Tp, num_heads * Dv, dtype=q.dtype, device=q.device)
+    assert out.shape == (Tp, num_heads * Dv) and out.is_contiguous()
+    rc = _hl().lig_paged_attention_mixed_heads_tiles(
+        _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(dist_bias),
+        0 if dist_bias is None else dist_bias.shape[0], _ptr(talk), _ptr(tile_seq),
+        _ptr(tile_qstart), _ptr(query_start_locs), _ptr(context_lens), _ptr(block_tables),
+        float(scale), int(chunk), tile_seq.shape[0], num_heads, G, D, Dv, bs,
+        block_tables.shape[1], _stream(),
+    )
+    return out if rc == 0 else None
+
+
 def token_shift_mix(x, mu, state, tok_seq, seg_start, seg_len, seg_slot, seg_fresh) -> torch.Tensor:
     """Several blends of every row with the row before it, from one pass:
     out[m] = x + (x_prev - x) * mu[m], x fp32 [R, W], mu [n, W] -> [n, R, W]
@@ -1015,21 +1067,22 @@ def token_shift_mix(x, mu, state, tok_seq, seg_start, seg_len, seg_slot, seg_fre
     return torch_ref.token_shift_mix(x, mu, state, seg_start, seg_len, seg_slot, seg_fresh, mu.dtype)
 
 
-MATRIX_STATE_KEY_SPLIT = 4
 # key channels per thread the scan kernel is instantiated for
 MATRIX_STATE_KEY_CLASSES = (4, 8, 12, 16, 24, 32, 48, 64)
 
 
 def matrix_state_width(heads: int, dim: int, vdim: int) -> int:
     """fp32 entries of one sequence's matrix state: the scan kernel splits a
-    head's key channels over four lanes and keeps the state in the order its
-    threads hold it, key channels padded to four times the kernel's size
-    class."""
-    need = (dim + MATRIX_STATE_KEY_SPLIT - 1) // MATRIX_STATE_KEY_SPLIT
+    head's key channels over 8 lanes (heads of 32 or more key channels whose
+    8 * vdim threads fit a workgroup) or 4, and keeps the state in the order
+    its threads hold it, key channels padded to the split times the kernel's
+    size class."""
+    split = 8 if dim >= 32 and vdim * 8 <= 1024 else 4
+    need = (dim + split - 1) // split
     kpt = next((c for c in MATRIX_STATE_KEY_CLASSES if c >= need), None)
     if kpt is None:
         raise ValueError(f"matrix-state heads hold at most 256 key channels, got {dim}")
-    return heads * MATRIX_STATE_KEY_SPLIT * kpt * vdim
+    return heads * split * kpt * vdim
 
 
 def matrix_state_scan(

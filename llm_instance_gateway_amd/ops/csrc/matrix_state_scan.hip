@@ -10,29 +10,30 @@
 //   optional silu on q, k, v as they are read.
 //
 // One workgroup per (segment, head).  A thread owns value column j and one
-// quarter of the key channels (lane = 4 j + s, keys s*KPT .. s*KPT + KPT-1,
-// KPT one of a few size classes),
-// keeps its KPT state entries in registers for the whole segment, and the
-// four partial outputs of a column are summed with two lane shuffles.  The
+// SPLIT-th of the key channels (lane = SPLIT j + s, keys s*KPT .. s*KPT +
+// KPT-1, KPT one of a few size classes; SPLIT is 8 for heads of 32 or more
+// key channels when 8 Dv threads fit a workgroup, else 4), keeps its KPT
+// state entries in registers for the whole segment, and the partial outputs
+// of a column are summed with lane shuffles.  The
 // segment is walked serially, TT tokens staged into LDS at a time (q, k, the
 // decay already exponentiated, v), so a prompt portion and a single decoded
 // token take the same arithmetic path in the same order: results do not
 // depend on how a sequence is cut into steps.
 //
 // The state row of a sequence is stored in the order the threads hold it,
-// [head][ii][thread] with D padded to 4*KPT: loads and stores are coalesced
-// (a row holds H * 4 * KPT * Dv entries; ops.matrix_state_width mirrors this).
+// [head][ii][thread] with D padded to SPLIT*KPT: loads and stores are
+// coalesced (a row holds H * SPLIT * KPT * Dv entries; ops.matrix_state_width
+// mirrors this).
 // A segment that starts its sequence ignores what the slot held.
 
 #include "elem_types.h"
 
-#define MS_SPLIT 4
 
-// KPT: key channels per thread (D is padded to 4 * KPT; padded channels carry
+// KPT: key channels per thread (D is padded to SPLIT * KPT; padded channels carry
 // q = k = w = 0 and stay zero).  MAXT bounds the workgroup size (4 * Dv
 // rounded up to whole waves) so the compiler may use the register file a
 // small workgroup leaves it.
-template <typename T, int KPT, bool BONUS, int MAXT>
+template <typename T, int MS_SPLIT, int KPT, bool BONUS, int MAXT>
 __global__ __launch_bounds__(MAXT) void matrix_state_scan_kernel(
     float* __restrict__ out,  // [R, H*Dv]
     const T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
@@ -102,7 +103,7 @@ __global__ __launch_bounds__(MAXT) void matrix_state_scan_kernel(
     __syncthreads();
     // every wave of the workgroup walks the tile (idle lanes of the last
     // wave take part in the shuffles with zeros)
-#pragma nounroll
+#pragma unroll 2
     for (int t = 0; t < nt_tok; ++t) {
       const float vj = owner ? v_s[t * Dv + j] : 0.f;
       const float* qt = q_s + t * Dp + s * KPT;
@@ -130,6 +131,7 @@ __global__ __launch_bounds__(MAXT) void matrix_state_scan_kernel(
       }
       o += __shfl_xor(o, 1, WAVE_SIZE);
       o += __shfl_xor(o, 2, WAVE_SIZE);
+      if (MS_SPLIT == 8) o += __shfl_xor(o, 4, WAVE_SIZE);
       if (owner && s == 0) out[(long)(r0 + t0 + t) * (H * Dv) + h * Dv + j] = o;
     }
   }
@@ -139,14 +141,19 @@ __global__ __launch_bounds__(MAXT) void matrix_state_scan_kernel(
   }
 }
 
-// Key channels per thread for a head of D key channels: the smallest size
-// class that holds ceil(D / 4); 0 when D is too wide.
-static int ms_keys_per_thread(int D) {
+// Key split and key channels per thread for a head of D key channels and Dv
+// value channels: the smallest size class that holds ceil(D / split); kpt 0
+// when D is too wide.
+static void ms_shape(int D, int Dv, int* split, int* kpt) {
   static const int classes[] = {4, 8, 12, 16, 24, 32, 48, 64};
-  const int need = (D + MS_SPLIT - 1) / MS_SPLIT;
+  *split = (D >= 32 && Dv * 8 <= 1024) ? 8 : 4;
+  const int need = (D + *split - 1) / *split;
+  *kpt = 0;
   for (int c : classes)
-    if (c >= need) return c;
-  return 0;
+    if (c >= need) {
+      *kpt = c;
+      break;
+    }
 }
 
 // Returns 0 when launched, 1 when a head is wider than the kernel holds.
@@ -156,37 +163,49 @@ extern "C" int lig_matrix_state_scan(
     const float* bonus, float* state, long state_stride, const int* seg_start,
     const int* seg_len, const int* seg_slot, const int* seg_fresh, int S, int H,
     int D, int Dv, int act_silu, int is_f32, hipStream_t stream) {
-  const int kpt = D > 0 ? ms_keys_per_thread(D) : 0;
+  int split = 4, kpt = 0;
+  if (D > 0) ms_shape(D, Dv, &split, &kpt);
   if (kpt == 0 || Dv <= 0 || Dv > 256) return 1;
   if (S <= 0) return 0;
-  const int Dp = kpt * MS_SPLIT;
+  const int Dp = kpt * split;
   const bool has_bonus = bonus != nullptr;
   const int per_tok = (has_bonus ? 3 : 2) * Dp + Dv;
   const int TT = per_tok * 16 * 4 <= 48 * 1024 ? 16 : 8;
   const size_t smem = (size_t)per_tok * TT * sizeof(float);
-  const int threads = ((Dv * MS_SPLIT + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE;
+  const int threads = ((Dv * split + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE;
   dim3 grid(S, H), block(threads);
-#define LIG_MS_T(T, KPT, B, MAXT)                                               \
-  hipLaunchKernelGGL((matrix_state_scan_kernel<T, KPT, B, MAXT>), grid, block,  \
-                     smem, stream, out, (const T*)q, q_stride, (const T*)k,     \
-                     k_stride, (const T*)v, v_stride, decay_pre, head_decay,    \
-                     bonus, state, state_stride, seg_start, seg_len, seg_slot,  \
-                     seg_fresh, H, D, Dv, TT, act_silu)
-#define LIG_MS(T, KPT, B)                               \
-  do {                                                  \
-    if (threads <= 256) LIG_MS_T(T, KPT, B, 256);       \
-    else LIG_MS_T(T, KPT, B, 1024);                     \
+#define LIG_MS_T(T, SP, KPT, B, MAXT)                                           \
+  hipLaunchKernelGGL((matrix_state_scan_kernel<T, SP, KPT, B, MAXT>), grid,     \
+                     block, smem, stream, out, (const T*)q, q_stride,           \
+                     (const T*)k, k_stride, (const T*)v, v_stride, decay_pre,   \
+                     head_decay, bonus, state, state_stride, seg_start,         \
+                     seg_len, seg_slot, seg_fresh, H, D, Dv, TT, act_silu)
+#define LIG_MS(T, SP, KPT, B)                             \
+  do {                                                    \
+    if (threads <= 256) LIG_MS_T(T, SP, KPT, B, 256);     \
+    else LIG_MS_T(T, SP, KPT, B, 1024);                   \
   } while (0)
-#define LIG_MS_K(T, B)                          \
-  switch (kpt) {                                \
-    case 4: LIG_MS(T, 4, B); break;             \
-    case 8: LIG_MS(T, 8, B); break;             \
-    case 12: LIG_MS(T, 12, B); break;           \
-    case 16: LIG_MS(T, 16, B); break;           \
-    case 24: LIG_MS(T, 24, B); break;           \
-    case 32: LIG_MS(T, 32, B); break;           \
-    case 48: LIG_MS(T, 48, B); break;           \
-    default: LIG_MS(T, 64, B); break;           \
+#define LIG_MS_K(T, B)                                    \
+  if (split == 8) {                                       \
+    switch (kpt) {                                        \
+      case 4: LIG_MS(T, 8, 4, B); break;                  \
+      case 8: LIG_MS(T, 8, 8, B); break;                  \
+      case 12: LIG_MS(T, 8, 12, B); break;                \
+      case 16: LIG_MS(T, 8, 16, B); break;                \
+      case 24: LIG_MS(T, 8, 24, B); break;                \
+      default: LIG_MS(T, 8, 32, B); break;                \
+    }                                                     \
+  } else {                                                \
+    switch (kpt) {                                        \
+      case 4: LIG_MS(T, 4, 4, B); break;                  \
+      case 8: LIG_MS(T, 4, 8, B); break;                  \
+      case 12: LIG_MS(T, 4, 12, B); break;                \
+      case 16: LIG_MS(T, 4, 16, B); break;                \
+      case 24: LIG_MS(T, 4, 24, B); break;                \
+      case 32: LIG_MS(T, 4, 32, B); break;                \
+      case 48: LIG_MS(T, 4, 48, B); break;                \
+      default: LIG_MS(T, 4, 64, B); break;                \
+    }                                                     \
   }
   if (is_f32) {
     if (has_bonus) { LIG_MS_K(float, true) } else { LIG_MS_K(float, false) }

@@ -32,7 +32,7 @@ SOURCES = [
     "group_norm.hip", "xielu.hip", "mingru.hip", "attention_general.hip",
     "attention_prefill_tiles.hip", "shift_norm.hip", "latent_attention.hip", "ff_act.hip",
     "attention_latent_rows.hip", "post_norm.hip", "qkv_prep.hip", "attention_mixed_heads.hip",
-    "matrix_state_scan.hip",
+    "matrix_state_scan.hip", "attention_mixed_heads_tiles.hip",
 ]
 SO_PATH = PKG / "_hybrid.so"
 
@@ -112,6 +112,9 @@ def _declare(lib: ctypes.CDLL) -> None:
     mh = lib.lig_paged_attention_mixed_heads
     mh.argtypes = [p, p, l, p, p, p, i, p, p, p, i, p, f, i, i, i, i, i, i, i, i, p]
     mh.restype = ctypes.c_int
+    mt = lib.lig_paged_attention_mixed_heads_tiles
+    mt.argtypes = [p, p, l, p, p, p, i, p, p, p, p, p, p, f, i, i, i, i, i, i, i, i, p]
+    mt.restype = ctypes.c_int
     ms = lib.lig_matrix_state_scan
     ms.argtypes = [p, p, l, p, l, p, l, p, p, p, p, l, p, p, p, p, i, i, i, i, i, i, p]
     ms.restype = ctypes.c_int

@@ -250,6 +250,56 @@ def test_mixed_heads_attention(device, dtype, H, G, D, chunk, rows_far):
     close(plain, want0[rows].reshape(len(rows), H * D), dtype)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("chunk,H,G,D", [(0, 4, 2, 16), (50, 6, 3, 48), (64, 16, 4, 64), (33, 1, 1, 24), (200, 12, 4, 128), (200, 12, 12, 128)])
+def test_mixed_heads_prompt_tiles(chunk, H, G, D):
+    """The MFMA head-mixing kernel: three portions in one launch (a whole
+    prompt, a portion that starts inside a chunk, a short one), chunk edges
+    inside and at the borders of its 16-row workgroups, a steep last bias row
+    and a mixing matrix far from the identity."""
+    dev, dtype = "cuda:0", torch.bfloat16
+    assert ops.mixed_heads_tiles_supported(dtype, D, D, H, True)
+    g = torch.Generator().manual_seed(9)
+    bs, scale, n_rel, far = 16, 0.4, 12, 90.0
+    c = chunk or 10 ** 6
+    rel = rnd(g, n_rel, H, s=0.8)
+    rel[-1] += 2.0
+    talk = torch.eye(H) + 0.4 * rnd(g, H, H)
+    tab = ops.distance_bias_table(rel.to(dev), far)
+    seqs = [(230, 0), (200, 90), (40, 37)]  # (tokens after the step, tokens before it)
+    kc, vc = make_caches(40, G, bs, D, D, dtype, dev)
+    qs, wants, tables, at = [], [], [], 0
+    for ctx, done in seqs:
+        plant = [(ctx - 1, ((ctx - 1) // c) * c), (ctx - 1, max(((ctx - 1) // c) * c - 1, 0)), (done, done),
+                 (done + 1, (done // c) * c), (min(done + 16, ctx - 1), done + 15 if done + 15 < ctx else done)]
+        q, k, v = planted(g, ctx, H, G, D, D, dtype, plant)
+        nb = (ctx + bs - 1) // bs
+        table = list(range(at, at + nb))[::-1]
+        at += nb
+        paged_sequence(k, v, bs, table, kc, vc)
+        want = O.chunked_attention(
+            q.double().numpy(), k.double().numpy(), v.double().numpy(), scale, chunk,
+            bias=O.distance_bias(rel.double().numpy(), ctx, far), talk=talk.double().numpy())
+        qs.append(q[done:].reshape(ctx - done, H * D))
+        wants.append(torch.from_numpy(want[done:].reshape(ctx - done, H * D)))
+        tables.append(table + [0] * (16 - nb))
+    lens = [c_ - d_ for c_, d_ in seqs]
+    qsl = [0, lens[0], lens[0] + lens[1], sum(lens)]
+    ts, tq = [], []
+    for si, n in enumerate(lens):
+        for qb in range(0, n, 64):
+            ts.append(si)
+            tq.append(qb)
+    got = ops.paged_attention_mixed_heads_tiles(
+        torch.cat(qs).to(dev), kc, vc, i32(tables, dev), i32(qsl, dev), i32([s_[0] for s_ in seqs], dev),
+        i32(ts, dev), i32(tq, dev), scale, H, dist_bias=tab, talk=talk.to(dev), chunk=chunk,
+    )
+    if G * D > 1024:  # K and V tiles of every key/value head exceed the LDS budget
+        assert got is None
+        return
+    close(got, torch.cat(wants), dtype)
+
+
 @pytest.mark.parametrize("device,dtype", CASES)
 def test_token_shift_mix_through_reused_slots(device, dtype):
     g = torch.Generator().manual_seed(6)
