@@ -4,7 +4,7 @@ through the engine, and the new kernels beside the like kernels of the
 Tikarax path against the HBM roofline.
 
     python bench.py --postnorm                  # both parts, JSON lines
-    python benchmarks/bench_postnorm.py --part engine|kernels [--sizes s,m]
+    python benchmarks/bench_postnorm.py --part engine|kernels|profile [--sizes s,m]
 
 Tikarax is the closest existing family: a hybrid stack whose layers
 alternate between paged attention of general head sizes and a recurrence
@@ -249,6 +249,12 @@ def main(argv=None) -> None:
         part_kernels(sizes)
     if "engine" in args.part:
         part_engine(sizes)
+    if "profile" in args.part:
+        # Potatar only: the run to put under a profiler
+        for name in sizes:
+            print(json.dumps({"bench": "profile", "size": name,
+                              "potatar": engine_run(potatar_config(name, SIZES[name]), 16, 1024, 64)}),
+                  flush=True)
 
 
 if __name__ == "__main__":

@@ -123,7 +123,7 @@ class PotatarLayer(nn.Module):
         elif spec.type == "wkv":
             self.mixer = MatrixStateMixer(
                 hidden, "wkv", m["heads"], m["dim"], m["dim"], eps,
-                decay_rank=int(m.get("decay_rank", 16)), device=device, dtype=dtype,
+                decay_rank=int(m.get("decay_rank", 32)), device=device, dtype=dtype,
             )
         else:
             lm, rm = m["left"], m["right"]
@@ -131,7 +131,7 @@ class PotatarLayer(nn.Module):
                 hidden, lm["heads"], lm["kv_heads"], lm["dim"], lm.get("vdim", lm["dim"]),
                 lm["scale"], eps, qk_norm="head", rot_dims=0,
                 chunk=int((lm.get("mask") or {}).get("size", 0)), values="key", bias=True,
-                dist_rows=int(lm.get("bias_rows", 16)), dist_far=float(lm["bias_max"]),
+                dist_rows=int(lm.get("bias_rows", 32)), dist_far=float(lm["bias_max"]),
                 talk=True, device=device, dtype=dtype,
             )
             self.right = MatrixStateMixer(

@@ -15,7 +15,7 @@
 // key channels when 8 Dv threads fit a workgroup, else 4), keeps its KPT
 // state entries in registers for the whole segment, and the partial outputs
 // of a column are summed with lane shuffles.  The
-// segment is walked serially, TT tokens staged into LDS at a time (q, k, the
+// segment is walked serially, TT (8 to 32) tokens staged into LDS at a time (q, k, the
 // decay already exponentiated, v), so a prompt portion and a single decoded
 // token take the same arithmetic path in the same order: results do not
 // depend on how a sequence is cut into steps.
@@ -28,6 +28,23 @@
 
 #include "elem_types.h"
 
+
+// Sum over the 4 or 8 neighbouring lanes that share a value column, through
+// the data-parallel lane permutes of the vector ALU (no trip through LDS):
+// swaps inside pairs, then pairs inside quads, then the two quads of a group
+// of 8 mirrored onto each other.
+template <int CTRL>
+LIG_DEVICE float lane_permute(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int SPLIT>
+LIG_DEVICE float split_sum(float o) {
+  o += lane_permute<0xB1>(o);   // quad_perm [1, 0, 3, 2]
+  o += lane_permute<0x4E>(o);   // quad_perm [2, 3, 0, 1]
+  if (SPLIT == 8) o += lane_permute<0x141>(o);  // row_half_mirror: lane i <-> 7 - i
+  return o;
+}
 
 // KPT: key channels per thread (D is padded to SPLIT * KPT; padded channels carry
 // q = k = w = 0 and stay zero).  MAXT bounds the workgroup size (4 * Dv
@@ -102,9 +119,9 @@ __global__ __launch_bounds__(MAXT) void matrix_state_scan_kernel(
     }
     __syncthreads();
     // every wave of the workgroup walks the tile (idle lanes of the last
-    // wave take part in the shuffles with zeros)
-#pragma unroll 2
-    for (int t = 0; t < nt_tok; ++t) {
+    // wave take part in the lane permutes with zeros)
+    // one token: read its q, k, decay and v from LDS, output, state update
+    auto step = [&](int t) __attribute__((always_inline)) {
       const float vj = owner ? v_s[t * Dv + j] : 0.f;
       const float* qt = q_s + t * Dp + s * KPT;
       const float* kt = k_s + t * Dp + s * KPT;
@@ -129,11 +146,18 @@ __global__ __launch_bounds__(MAXT) void matrix_state_scan_kernel(
           }
         }
       }
-      o += __shfl_xor(o, 1, WAVE_SIZE);
-      o += __shfl_xor(o, 2, WAVE_SIZE);
-      if (MS_SPLIT == 8) o += __shfl_xor(o, 4, WAVE_SIZE);
+      o = split_sum<MS_SPLIT>(o);
       if (owner && s == 0) out[(long)(r0 + t0 + t) * (H * Dv) + h * Dv + j] = o;
+    };
+    // two tokens per trip: the second token's LDS reads overlap the first
+    // token's arithmetic (the state update itself stays in order)
+    int t = 0;
+#pragma nounroll
+    for (; t + 1 < nt_tok; t += 2) {
+      step(t);
+      step(t + 1);
     }
+    if (t < nt_tok) step(t);
   }
   if (owner) {
 #pragma unroll
@@ -170,7 +194,8 @@ extern "C" int lig_matrix_state_scan(
   const int Dp = kpt * split;
   const bool has_bonus = bonus != nullptr;
   const int per_tok = (has_bonus ? 3 : 2) * Dp + Dv;
-  const int TT = per_tok * 16 * 4 <= 48 * 1024 ? 16 : 8;
+  // tokens staged per tile: as many as 40 KB of LDS hold, 8 to 32
+  const int TT = per_tok * 32 * 4 <= 40 * 1024 ? 32 : (per_tok * 16 * 4 <= 48 * 1024 ? 16 : 8);
   const size_t smem = (size_t)per_tok * TT * sizeof(float);
   const int threads = ((Dv * split + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE;
   dim3 grid(S, H), block(threads);
