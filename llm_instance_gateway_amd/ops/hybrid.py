@@ -1,5 +1,6 @@
 """Light native library for the hybrid-model kernels (grouped RMS norm, xIELU,
-minGRU scan, general-size paged attention).
+minGRU scan, general-size paged attention, shift norms, latent attention,
+sum+norm residual step, q/k/v prep, head-mixed attention, matrix-state scan).
 
 These kernels expose a plain C ABI and need no torch headers, so they are
 compiled by one direct ``hipcc -shared`` call (seconds, not the minutes the

@@ -447,3 +447,38 @@ def test_graph_decode_matches_eager(model_a):
         eng.generate_all(max_steps=100)
         outs.append([s.output_token_ids for s in seqs])
     assert outs[0] == outs[1]
+
+
+def test_served_through_the_pool_and_front_door(tmp_path):
+    """A model folder as the pool's base model: worker process, router, HTTP
+    front door, greedy completion from prompt token ids."""
+    from starlette.testclient import TestClient
+
+    from llm_instance_gateway_amd.api.types import InferenceModel
+    from llm_instance_gateway_amd.serving import EnginePool, build_app
+
+    cfg = dict(CFG_A, vocab=300)
+    W = make_checkpoint(cfg, 24)
+    path = write_model(tmp_path / "served", cfg, W)
+    pool = EnginePool(
+        path, devices=["cpu"],
+        engine_kwargs=dict(num_kv_blocks=64, max_num_seqs=4, max_num_batched_tokens=64, max_model_len=256),
+    )
+    pool.start()
+    try:
+        pool.datastore.store_model(InferenceModel(model_name="postnorm"))
+        client = TestClient(build_app(pool))
+        prompt = tokens_for(cfg, 23, 8)
+        r = client.post("/v1/completions", json={"model": "postnorm", "prompt": prompt, "max_tokens": 5})
+        assert r.status_code == 200, r.text
+        out = r.json()["choices"][0]["token_ids"]
+        assert len(out) == 5
+        toks = list(prompt)
+        for step in range(5):  # workers run bf16: only a clear argmax must match
+            logits = oracle(cfg, W, toks)[0][-1]
+            top2 = torch.topk(logits, 2).values
+            if float(top2[0] - top2[1]) > 0.2:
+                assert out[step] == int(torch.argmax(logits)), (step, out)
+            toks.append(out[step])
+    finally:
+        pool.stop()
