@@ -996,7 +996,8 @@ def paged_attention_mixed_heads(
 
 def mixed_heads_tiles_supported(q_dtype, k_dim: int, v_dim: int, heads: int, is_cuda: bool) -> bool:
     """The MFMA head-mixing kernel for prompt rows: bf16, head sizes multiples
-    of 8 up to 128, at most 16 heads (one wave per head in a workgroup)."""
+    of 8 up to 128, at most 32 heads (a workgroup holds all heads: one wave
+    per head up to 16, two heads per wave beyond)."""
     return (
         is_cuda
         and q_dtype == torch.bfloat16
@@ -1004,7 +1005,7 @@ def mixed_heads_tiles_supported(q_dtype, k_dim: int, v_dim: int, heads: int, is_
         and v_dim % 8 == 0
         and 0 < k_dim <= 128
         and 0 < v_dim <= 128
-        and 1 <= heads <= 16
+        and 1 <= heads <= 32
         and os.environ.get("LIG_FORCE_TORCH_OPS") != "1"
         and os.environ.get("LIG_GENERAL_ATTENTION") != "1"
     )

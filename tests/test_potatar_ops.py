@@ -251,12 +251,14 @@ def test_mixed_heads_attention(device, dtype, H, G, D, chunk, rows_far):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("chunk,H,G,D", [(0, 4, 2, 16), (50, 6, 3, 48), (64, 16, 4, 64), (33, 1, 1, 24), (200, 12, 4, 128), (200, 12, 12, 128)])
+@pytest.mark.parametrize("chunk,H,G,D", [(0, 4, 2, 16), (50, 6, 3, 48), (64, 16, 4, 64), (33, 1, 1, 24), (200, 12, 4, 128), (200, 12, 12, 128),
+                                           (64, 32, 8, 64), (50, 20, 5, 32)])
 def test_mixed_heads_prompt_tiles(chunk, H, G, D):
     """The MFMA head-mixing kernel: three portions in one launch (a whole
     prompt, a portion that starts inside a chunk, a short one), chunk edges
     inside and at the borders of its 16-row workgroups, a steep last bias row
-    and a mixing matrix far from the identity."""
+    and a mixing matrix far from the identity; up to 16 heads a wave serves
+    one head, beyond that two."""
     dev, dtype = "cuda:0", torch.bfloat16
     assert ops.mixed_heads_tiles_supported(dtype, D, D, H, True)
     g = torch.Generator().manual_seed(9)
