@@ -17,7 +17,7 @@ from typing import Any, Dict, List, Optional, Tuple
 @dataclass
 class LayerSpec:
     """One layer of a heterogeneous (hybrid) stack: which sequence mixer it
-    has ('attention' keeps paged K/V, 'mingru' keeps a recurrent state
+    has ('attention' and 'attention_2' keep paged K/V, 'mingru' keeps a recurrent state
     vector), the mixer's sizes and constants, and its feed-forward (None for
     a layer without one).  'latent_attention' keeps one paged row per token
     (the normalised key/value latent followed by the shared rotated key
@@ -72,6 +72,13 @@ class ModelConfig:
     residual_alpha: float = 1.0
     # logits <- cap * tanh(logits / cap); 0 = no cap.
     logit_softcap: float = 0.0
+    # Pre-norm stacks with a scaled branch: x <- x + residual_mult * sublayer(norm(x)).
+    residual_mult: float = 1.0
+    # The residual as several parallel streams that sub-layers read through a
+    # weighted sum and write through a mixing matrix (hyper_connections);
+    # one stream without them is the ordinary residual.
+    residual_streams: int = 1
+    hyper_connections: bool = False
 
     @property
     def is_moe(self) -> bool:
@@ -100,7 +107,7 @@ class ModelConfig:
         total = 0
         for i in self.layer_run_order():
             s = self.layer_specs[i]
-            if s.type == "attention":
+            if s.type in ("attention", "attention_2"):
                 total += (s.mixer["kv_heads"] // tp_size) * (s.mixer["dim"] + s.mixer["vdim"])
             elif s.type == "latent_attention":
                 total += s.mixer["kv_rank"] + s.mixer["rot_dim"]

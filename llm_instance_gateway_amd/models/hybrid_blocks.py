@@ -12,6 +12,15 @@ arguments, so another model family can assemble them differently.
   * `MinGRU` — the minimal gated recurrent unit: gates read only the current
     token, the state is an fp32 vector per sequence in a slot pool.
   * `XieluMLP` — two-matrix feed-forward with the xIELU activation.
+  * `LatentAttention`, `ReluSquaredMLP`, `ScoredExpertsMLP` — low-rank
+    key/value attention and its feed-forwards.
+  * `NormedRotaryAttention` — q/k norms before or after a partial rotation in
+    either pair layout, chunked or sliding-window visibility, softmax (with
+    an optional sink) or unnormalised sigmoid weights, distance bias, head
+    mixing, per-head output gate.
+  * `MatrixStateMixer`, `GeluMLP` — matrix-state recurrences.
+  * `GatedReluMLP`, `GroupRoutedExpertsMLP` — gated feed-forward and routed
+    experts with a softmax router, group-limited choice and identity experts.
 
 Projections are library GEMMs over fused weights (one GEMM in, one out per
 block); everything between them is one HIP kernel each (ops layer).
@@ -440,9 +449,19 @@ class NormedRotaryAttention(nn.Module):
 
       * qk_norm "row": one norm over the whole q (and k) projection with
         weights of that size; "head": per head with one weight of size dim
-        shared by the heads; "none".
-      * rot_dims entries of every head are rotated (pairs i, i + rot_dims/2);
+        shared by the heads; "head_post": per head AFTER the rotation, no
+        weights; "none".
+      * rot_dims entries of every head are rotated; rot_layout "half" pairs
+        entry i with i + rot_dims/2, "interleaved" pairs 2i with 2i + 1;
+        rot_scale divides every frequency (linear position scaling);
         0 = no rotation.
+      * window: a query sees itself and the window - 1 tokens before it
+        (0 = no window; may be combined with chunk).
+      * weights "softmax", optionally with a zero-score sink in the
+        denominator (sink=True), or "sigmoid": every visible key weighs
+        sigmoid(score + score_bias[head]), nothing is normalised.
+      * head_gate: head h's output is multiplied by sigmoid(W_g x)_h, one
+        number per head; the gate rows ride in the fused input GEMM.
       * values "proj": a projection of their own; "key": the keys as
         projected, before their norm (no value weights).
       * v_unit_norm: every head's value is divided by its root mean square.
@@ -465,10 +484,15 @@ class NormedRotaryAttention(nn.Module):
         eps: float, qk_norm: str = "row", rot_base: float = 10000.0, rot_dims: int = 0,
         chunk: int = 0, values: str = "proj", v_unit_norm: bool = False, bias: bool = True,
         dist_rows: int = 0, dist_far: float = 0.0, talk: bool = False,
-        device="cpu", dtype=torch.bfloat16,
+        rot_layout: str = "half", rot_scale: float = 1.0, window: int = 0,
+        weights: str = "softmax", score_bias: bool = False, sink: bool = False,
+        head_gate: bool = False, device="cpu", dtype=torch.bfloat16,
     ) -> None:
         super().__init__()
-        assert heads % kv_heads == 0 and qk_norm in ("none", "row", "head")
+        assert heads % kv_heads == 0 and qk_norm in ("none", "row", "head", "head_post")
+        assert rot_layout in ("half", "interleaved") and weights in ("softmax", "sigmoid")
+        assert not (score_bias and weights != "sigmoid") and not (sink and weights != "softmax")
+        assert not ((dist_rows > 0 or talk) and (window > 0 or weights == "sigmoid" or sink or head_gate))
         assert values in ("proj", "key") and (values == "proj" or vdim == dim)
         assert 0 <= rot_dims <= dim and rot_dims % 2 == 0
         self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
@@ -477,11 +501,27 @@ class NormedRotaryAttention(nn.Module):
         self.nq, self.nk = heads * dim, kv_heads * dim
         self.nv = kv_heads * vdim if values == "proj" else 0
         self.n_in = self.nq + self.nk + self.nv
+        self.window, self.weights, self.rot_layout = int(window), weights, rot_layout
+        # gate rows follow q | k | v; the fused weight is padded with zero rows
+        # to a multiple of 8 so that rows of the projection stay 16-byte aligned
+        self.n_gate = heads if head_gate else 0
+        n_rows = (self.n_in + self.n_gate + 7) // 8 * 8 if head_gate else self.n_in
         s = 1.0 / math.sqrt(hidden)
-        self.w_in = _param((self.n_in, hidden), device, dtype, s)
-        self.b_in = _param((self.n_in,), device, dtype, 0.1 if bias else None)
+        self.w_in = _param((n_rows, hidden), device, dtype, s)
+        self.b_in = _param((n_rows,), device, dtype, 0.1 if bias else None)
+        with torch.no_grad():
+            self.w_in[self.n_in + self.n_gate :].zero_()
+            self.b_in[self.n_in :].zero_()
         self.has_bias = bias
-        nw = {"row": (self.nq, self.nk), "head": (dim, dim), "none": (0, 0)}[qk_norm]
+        # fp32 whatever the activation dtype: they enter the scores
+        self.score_bias = (
+            nn.Parameter(torch.empty(heads, device=device).uniform_(-1.0, 1.0), requires_grad=False)
+            if score_bias else None
+        )
+        self.sink = (
+            nn.Parameter(torch.zeros(heads, device=device), requires_grad=False) if sink else None
+        )
+        nw = {"row": (self.nq, self.nk), "head": (dim, dim), "none": (0, 0), "head_post": (0, 0)}[qk_norm]
         self.q_norm = _param((nw[0],), device, dtype, None)
         self.k_norm = _param((nw[1],), device, dtype, None)
         with torch.no_grad():
@@ -507,7 +547,7 @@ class NormedRotaryAttention(nn.Module):
         self.refresh_tables()
         self.register_buffer(
             "inv_freq",
-            ops.rotary_inv_freq(rot_base, rot_dims, device) if rot_dims > 0 else None,
+            ops.rotary_inv_freq(rot_base, rot_dims, device, rot_scale) if rot_dims > 0 else None,
             persistent=False,
         )
 
@@ -525,12 +565,19 @@ class NormedRotaryAttention(nn.Module):
 
     def load(self, get, prefix: str) -> None:
         names = ["q", "k"] + (["v"] if self.values == "proj" else [])
+        if self.n_gate:
+            names.append("g")
         with torch.no_grad():
-            self.w_in.copy_(torch.cat([get(prefix + n) for n in names], dim=0))
+            rows = torch.cat([get(prefix + n) for n in names], dim=0)
+            self.w_in.zero_()
+            self.w_in[: rows.shape[0]].copy_(rows)
             if self.has_bias:
-                self.b_in.copy_(torch.cat([get(prefix + n + ".b") for n in names], dim=0))
+                names_b = [n for n in names if n != "g"]
+                self.b_in[: self.n_in].copy_(torch.cat([get(prefix + n + ".b") for n in names_b], dim=0))
                 self.b_o.copy_(get(prefix + "o.b"))
-            if self.qk_norm != "none":
+            if self.score_bias is not None:
+                self.score_bias.copy_(get(prefix + "pb").float())
+            if self.qk_norm in ("row", "head"):
                 self.q_norm.copy_(get(prefix + "q.norm"))
                 self.k_norm.copy_(get(prefix + "k.norm"))
             self.w_o.copy_(get(prefix + "o"))
@@ -548,12 +595,13 @@ class NormedRotaryAttention(nn.Module):
             proj, self.heads, self.kv_heads, self.dim, self.vdim, self.qk_norm,
             self.q_norm, self.k_norm, self.eps, self.inv_freq, positions, k_cache, v_cache,
             meta.slot_mapping, v_source=self.values, v_unit_norm=self.v_unit_norm,
-            v_first=v_first, lam=self.lam, want_v=want_v,
+            v_first=v_first, lam=self.lam, want_v=want_v, rot_layout=self.rot_layout,
         )
         if self.mixes_heads:
             o = self._attend_mixed(q, positions, k_cache, v_cache, meta)
         else:
-            o = self._attend(q, positions, k_cache, v_cache, meta)
+            gate = proj[:, self.n_in : self.n_in + self.n_gate] if self.n_gate else None
+            o = self._attend(q, positions, k_cache, v_cache, meta, gate)
         y = F.linear(o, self.w_o, self.b_o if self.has_bias else None)
         return (y, v_out) if want_v else y
 
@@ -591,8 +639,12 @@ class NormedRotaryAttention(nn.Module):
         )
         return o
 
-    def _attend(self, q, positions, k_cache, v_cache, meta):
+    def _attend(self, q, positions, k_cache, v_cache, meta, gate=None):
         np_, rows = meta.num_prefill_tokens, q.shape[0]
+        kw = dict(
+            chunk=self.chunk, window=self.window, weights=self.weights,
+            score_bias=self.score_bias, sink=self.sink, gate_per_head=gate is not None,
+        )
         if (
             np_ > 0
             and meta.prefill_tile_seq is not None
@@ -605,17 +657,18 @@ class NormedRotaryAttention(nn.Module):
                 q[:np_], k_cache, v_cache, meta.prefill_block_tables,
                 meta.prefill_query_start_locs, meta.prefill_context_lens,
                 meta.prefill_tile_seq, meta.prefill_tile_qstart, self.scale, self.heads,
-                out=o[:np_], chunk=self.chunk,
+                out=o[:np_], gate=None if gate is None else gate[:np_], **kw,
             )
             if rows > np_:
                 ops.paged_attention_general(
                     q[np_:], k_cache, v_cache, meta.seq_block_tables, meta.tok_seq[np_:],
-                    positions[np_:], self.scale, self.heads, out=o[np_:], chunk=self.chunk,
+                    positions[np_:], self.scale, self.heads, out=o[np_:],
+                    gate=None if gate is None else gate[np_:], **kw,
                 )
             return o
         return ops.paged_attention_general(
             q, k_cache, v_cache, meta.seq_block_tables, meta.tok_seq, positions,
-            self.scale, self.heads, chunk=self.chunk,
+            self.scale, self.heads, gate=gate, **kw,
         )
 
 
@@ -750,3 +803,127 @@ class GeluMLP(nn.Module):
 
     def forward(self, h, meta=None):
         return _mm(ops.gelu_erf(_mm(h, self.w_up)), self.w_down)
+
+
+class GatedReluMLP(nn.Module):
+    """down(relu(gate h) * (up h)); gate and up are one fused GEMM."""
+
+    def __init__(self, hidden: int, ff: int, device="cpu", dtype=torch.bfloat16) -> None:
+        super().__init__()
+        self.w13 = _param((2 * ff, hidden), device, dtype, 1.0 / math.sqrt(hidden))
+        self.w_down = _param((hidden, ff), device, dtype, 1.0 / math.sqrt(ff))
+
+    def load(self, get, prefix: str) -> None:
+        with torch.no_grad():
+            self.w13.copy_(torch.cat([get(prefix + "gate"), get(prefix + "up")], dim=0))
+            self.w_down.copy_(get(prefix + "down"))
+
+    def forward(self, h, meta=None):
+        return _mm(ops.glu_act(_mm(h, self.w13), "relu"), self.w_down)
+
+
+def expert_dispatch_plan(idx: torch.Tensor, experts: int):
+    """Capacity-padded dispatch of (token, choice) pairs to `experts` batches.
+
+    idx int64 [T, top]; choices >= experts take part in no batch.  Returns
+    (gather [experts * cap] int64: the token of every batch row, -1 for
+    padding; rows [T, top] int64: the batch row of every pair, -1 for pairs
+    outside the batches; cap).  One host round trip (the capacity)."""
+    T, top = idx.shape
+    dev = idx.device
+    flat_e = idx.reshape(-1)
+    flat_t = torch.arange(T, device=dev).unsqueeze(1).expand(T, top).reshape(-1)
+    order = torch.argsort(flat_e, stable=True)
+    se, stok = flat_e[order], flat_t[order]
+    inside = se < experts
+    counts = torch.bincount(se.clamp(max=experts), minlength=experts + 1)
+    cap = max(int(counts[:experts].max()), 1)
+    starts = torch.cumsum(counts, 0) - counts
+    pos_in_e = torch.arange(se.numel(), device=dev) - starts.index_select(0, se.clamp(max=experts))
+    trash = experts * cap  # one spare row takes the pairs outside the batches
+    dest = torch.where(inside, se * cap + pos_in_e, torch.full_like(se, trash))
+    gather = torch.full((trash + 1,), -1, dtype=torch.int64, device=dev)
+    gather.index_copy_(0, dest, stok)
+    rows = torch.empty_like(dest)
+    rows[order] = torch.where(inside, dest, torch.full_like(dest, -1))
+    return gather[:trash], rows.view(T, top), cap
+
+
+class GroupRoutedExpertsMLP(nn.Module):
+    """Routed gated experts behind a softmax router with group-limited choice.
+
+    z = W_r h in fp32 over experts + identity outputs; scores softmax(z);
+    the choice adds a per-output correction and only looks at the `keep` best
+    of `groups` groups of neighbouring outputs (`ops.grouped_topk_route`);
+    the chosen plain scores, divided by their sum, weigh the experts'
+    OUTPUTS.  The last `identity` outputs are experts without weights whose
+    output is their input.  An expert is down(act(gate h, up h)) with
+    g = min(gate, limit), u = clamp(up, -limit, limit), act = g * sigmoid(alpha
+    g) * (u + 1).
+
+    Dispatch as `ScoredExpertsMLP`: pairs sorted by expert into a
+    capacity-padded [E, cap, hidden] batch and one batched GEMM pair; steps
+    of single tokens only let every expert see every token (static shapes,
+    no host round trip), the combine picks the chosen ones.
+    """
+
+    def __init__(
+        self, hidden: int, ff: int, experts: int, top: int, identity: int = 0,
+        groups: int = 1, keep: int = 1, limit: float = 7.0, alpha: float = 1.702,
+        device="cpu", dtype=torch.bfloat16,
+    ) -> None:
+        super().__init__()
+        n = experts + identity
+        assert experts >= 1 and identity >= 0 and n % groups == 0 and 1 <= keep <= groups
+        assert 1 <= top <= keep * (n // groups)
+        self.experts, self.identity, self.top, self.ff = experts, identity, top, ff
+        self.groups, self.keep = groups, keep
+        self.limit, self.alpha = float(limit), float(alpha)
+        # router and correction are fp32 whatever the activation dtype
+        self.w_router = nn.Parameter(
+            torch.empty(n, hidden, device=device, dtype=torch.float32).uniform_(
+                -1.0 / math.sqrt(hidden), 1.0 / math.sqrt(hidden)
+            ),
+            requires_grad=False,
+        )
+        self.correction = nn.Parameter(
+            torch.zeros(n, device=device, dtype=torch.float32), requires_grad=False
+        )
+        # pre-transposed for bmm: [E, hidden, gate | up] and [E, ff, hidden]
+        self.w13 = _param((experts, hidden, 2 * ff), device, dtype, 1.0 / math.sqrt(hidden))
+        self.w2 = _param((experts, ff, hidden), device, dtype, 1.0 / math.sqrt(ff))
+
+    def load(self, get, prefix: str, has=None) -> None:
+        with torch.no_grad():
+            self.w_router.copy_(get(prefix + "router").float())
+            if has is None or has(prefix + "correction"):
+                self.correction.copy_(get(prefix + "correction").float())
+            for e in range(self.experts):
+                p = f"{prefix}e{e}."
+                self.w13[e].copy_(torch.cat([get(p + "gate"), get(p + "up")], dim=0).t())
+                self.w2[e].copy_(get(p + "down").t())
+
+    def route(self, h: torch.Tensor):
+        z = F.linear(h.float(), self.w_router)
+        idx, w = ops.grouped_topk_route(z, self.correction, self.top, self.groups, self.keep)
+        return w, idx.long()
+
+    def _experts(self, xe: torch.Tensor, rows: int) -> torch.Tensor:
+        """xe [E, rows, hidden] -> [E * rows, hidden]."""
+        E = self.experts
+        act = ops.glu_act(torch.bmm(xe, self.w13).view(E * rows, -1), "clamped", self.limit, self.alpha)
+        return torch.bmm(act.view(E, rows, self.ff), self.w2).view(E * rows, -1)
+
+    def forward(self, h, meta=None):
+        T, hidden = h.shape
+        E = self.experts
+        w, idx = self.route(h)
+        if meta is not None and meta.num_prefill_tokens == 0:
+            ye = self._experts(h.unsqueeze(0).expand(E, T, hidden), T)
+            tok = torch.arange(T, device=h.device).unsqueeze(1)
+            rows = torch.where(idx < E, idx * T + tok, torch.full_like(idx, -1))
+            return ops.routed_combine(ye, h, rows.contiguous(), w)
+        gather, rows, cap = expert_dispatch_plan(idx, E)
+        xe = ops.scale_gather_rows(h, gather, (gather >= 0).float())
+        ye = self._experts(xe.view(E, cap, hidden), cap)
+        return ops.routed_combine(ye, h, rows.contiguous(), w)

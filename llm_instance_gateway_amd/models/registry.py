@@ -68,7 +68,20 @@ def _potatar_config(raw: dict, path: str) -> ModelConfig:
     return config_from_json(raw, path)
 
 
+def _vemenex_factory(cfg, device, dtype, tp):
+    from .vemenex import VemenexForCausalLM
+
+    return VemenexForCausalLM(cfg, device=device, dtype=dtype, tp=tp)
+
+
+def _vemenex_config(raw: dict, path: str) -> ModelConfig:
+    from .vemenex import config_from_json
+
+    return config_from_json(raw, path)
+
+
 register_architecture("llama", None, _llama_factory)
+register_architecture("vemenex", _vemenex_config, _vemenex_factory)
 register_architecture("potatar", _potatar_config, _potatar_factory)
 register_architecture("lopovik", _lopovik_config, _lopovik_factory)
 register_architecture("tikarax", _tikarax_config, _tikarax_factory)

@@ -481,7 +481,8 @@ def paged_attention_general(
     q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float,
     num_heads: int, gate=None, temp_coef: float = 0.0, temp_every: float = 1.0,
     out: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
-    chunk: int = 0,
+    chunk: int = 0, window: int = 0, score_bias: Optional[torch.Tensor] = None,
+    weights: str = "softmax", gate_per_head: bool = False,
 ) -> torch.Tensor:
     """Causal paged attention for any key/value head sizes; token r of the
     flat batch attends keys 0..positions[r] of sequence tok_seq[r].  Optional
@@ -489,7 +490,12 @@ def paged_attention_general(
     and per-head softmax sink (fp32 [heads]: exp(sink) joins the denominator).
     q/gate may be column-block views with a row stride; v_cache may be a view
     of the leading entries of k_cache's rows (a latent cache).  chunk > 0:
-    only keys of the query's own chunk, floor(j/chunk) == floor(p/chunk)."""
+    only keys of the query's own chunk, floor(j/chunk) == floor(p/chunk).
+    window > 0: only keys j with p - j < window.  weights "sigmoid": every
+    visible key weighs sigmoid(score + score_bias[head]) (fp32 [heads],
+    optional) and nothing is normalised.  gate_per_head: gate is [R, heads],
+    one logistic gate per head."""
+    assert weights in ("softmax", "sigmoid") and (weights == "sigmoid" or score_bias is None)
     if _use_hybrid(q):
         nb, G, bs, D = k_cache.shape
         Dv = v_cache.shape[-1]
@@ -502,7 +508,11 @@ def paged_attention_general(
         assert block_tables.dtype == torch.int32 and tok_seq.dtype == torch.int32
         assert positions.dtype == torch.int64 and block_tables.is_contiguous()
         if gate is not None:
-            assert gate.shape == (R, num_heads * Dv) and gate.stride(1) == 1
+            gcols = num_heads if gate_per_head else num_heads * Dv
+            assert gate.shape == (R, gcols) and gate.stride(1) == 1 and gate.dtype == q.dtype
+        if score_bias is not None:
+            assert score_bias.dtype == torch.float32 and score_bias.shape == (num_heads,)
+            assert score_bias.is_contiguous()
         if out is None:
             out = torch.empty(R, num_heads * Dv, dtype=q.dtype, device=q.device)
         assert out.shape == (R, num_heads * Dv) and out.is_contiguous() and out.dtype == q.dtype
@@ -513,12 +523,15 @@ def paged_attention_general(
             _ptr(block_tables), block_tables.shape[1], _ptr(tok_seq),
             _ptr(positions), _ptr(gate), 0 if gate is None else gate.stride(0),
             _ptr(sink), float(scale), float(temp_coef), ev, ev_int, R, num_heads,
-            G, D, Dv, v_row, bs, int(chunk), _is_f32(q), _stream(),
+            G, D, Dv, v_row, bs, int(chunk), int(window), _ptr(score_bias),
+            int(weights == "sigmoid"), int(bool(gate_per_head and gate is not None)),
+            _is_f32(q), _stream(),
         )
         return out
     res = torch_ref.paged_attention_general(
         q, k_cache, v_cache, block_tables, tok_seq, positions, scale, num_heads,
-        gate, temp_coef, temp_every, sink, chunk,
+        gate, temp_coef, temp_every, sink, chunk, window, score_bias, weights,
+        gate_per_head,
     )
     if out is not None:
         out.copy_(res)
@@ -580,7 +593,9 @@ def paged_attention_prefill_tiles(
     q, k_cache, v_cache, block_tables, query_start_locs, context_lens, tile_seq,
     tile_qstart, scale: float, num_heads: int, gate=None, temp_coef: float = 0.0,
     temp_every: float = 1.0, out: Optional[torch.Tensor] = None,
-    sink: Optional[torch.Tensor] = None, chunk: int = 0,
+    sink: Optional[torch.Tensor] = None, chunk: int = 0, window: int = 0,
+    score_bias: Optional[torch.Tensor] = None, weights: str = "softmax",
+    gate_per_head: bool = False,
 ) -> torch.Tensor:
     """Prompt-partition attention on MFMA tiles for any head sizes the kernel
     takes (`tiled_prefill_supported`): q [Tp, H*D] (strided view allowed) are
@@ -588,7 +603,10 @@ def paged_attention_prefill_tiles(
     context_lens count each sequence's tokens after this step; tile_seq /
     tile_qstart name the 64-row query tiles.  Temperature, sigmoid gate and
     softmax sink are fused; v_cache may view the head of k_cache's rows; chunk
-    > 0 restricts every row to the keys of its own chunk.  GPU only."""
+    > 0 restricts every row to the keys of its own chunk, window > 0 to the
+    last `window` keys up to its own.  weights "sigmoid", score_bias and
+    gate_per_head as in `paged_attention_general`.  GPU only."""
+    assert weights in ("softmax", "sigmoid") and (weights == "sigmoid" or score_bias is None)
     nb, G, bs, D = k_cache.shape
     Dv = v_cache.shape[-1]
     v_row = _value_row_stride(v_cache)
@@ -600,7 +618,11 @@ def paged_attention_prefill_tiles(
     for t in (block_tables, query_start_locs, context_lens, tile_seq, tile_qstart):
         assert t.dtype == torch.int32 and t.is_contiguous()
     if gate is not None:
-        assert gate.shape == (Tp, num_heads * Dv) and gate.stride(1) == 1
+        gcols = num_heads if gate_per_head else num_heads * Dv
+        assert gate.shape == (Tp, gcols) and gate.stride(1) == 1 and gate.dtype == q.dtype
+    if score_bias is not None:
+        assert score_bias.dtype == torch.float32 and score_bias.shape == (num_heads,)
+        assert score_bias.is_contiguous()
     if out is None:
         out = torch.empty(Tp, num_heads * Dv, dtype=q.dtype, device=q.device)
     assert out.shape == (Tp, num_heads * Dv) and out.is_contiguous()
@@ -612,7 +634,8 @@ def paged_attention_prefill_tiles(
         _ptr(tile_qstart), _ptr(query_start_locs), _ptr(context_lens),
         _ptr(block_tables), float(scale), float(temp_coef), ev, ev_int,
         tile_seq.shape[0], num_heads, G, D, Dv, v_row, bs, block_tables.shape[1],
-        int(chunk), _stream(),
+        int(chunk), int(window), _ptr(score_bias), int(weights == "sigmoid"),
+        int(bool(gate_per_head and gate is not None)), _stream(),
     )
     if rc != 0:
         raise RuntimeError("paged_attention_prefill_tiles: shape or alignment not served")
@@ -863,14 +886,14 @@ def scaled_add_rms_norm(
     return torch_ref.scaled_add_rms_norm(x, alpha, w, eps, y1, s1, y2, s2, w.dtype)
 
 
-_QK_NORM_MODES = {"none": 0, "row": 1, "head": 2}
+_QK_NORM_MODES = {"none": 0, "row": 1, "head": 2, "head_post": 3}
 
 
 def qkv_norm_rope_cache(
     proj, heads: int, kv_heads: int, dim: int, vdim: int, qk_norm: str, w_q, w_k,
     eps: float, inv_freq, positions, k_cache, v_cache, slot_mapping,
     v_source: str = "proj", v_unit_norm: bool = False, v_first=None, lam: float = 0.0,
-    want_v: bool = False,
+    want_v: bool = False, rot_layout: str = "half",
 ):
     """Everything between the fused input projection and the attention
     kernel, one pass per token row of proj = [q | k | v] (or [q | k] with
@@ -878,13 +901,16 @@ def qkv_norm_rope_cache(
 
     qk_norm "row": RMS norm over all of q (and of k) with weights of that
     size; "head": per head, one weight of size dim shared by the heads;
-    "none".  Then rotate-half rotation of the first 2*len(inv_freq) entries
-    of every q and k head (inv_freq None: no rotation).  Values: optionally
+    "none"; "head_post": per head AFTER the rotation, without weights.  The
+    rotation turns the first 2*len(inv_freq) entries of every q and k head
+    (inv_freq None: no rotation); rot_layout "half" pairs entry i with entry
+    i + len(inv_freq), "interleaved" pairs entry 2i with 2i + 1.  Values: optionally
     divided per head by their root mean square, optionally blended with
     v_first (fp32 [R, kv_heads*vdim]) as (1 - lam) v + lam v_first.  Keys and
     values go to the paged caches at slot_mapping; returns (q [R, heads*dim]
     contiguous, the values as cached in fp32 if want_v else None)."""
     mode = _QK_NORM_MODES[qk_norm]
+    assert rot_layout in ("half", "interleaved")
     from_key = v_source == "key"
     assert v_source in ("proj", "key") and (not from_key or vdim == dim)
     if _use_hybrid(proj):
@@ -908,16 +934,18 @@ def qkv_norm_rope_cache(
         q_out = torch.empty(R, nq, dtype=proj.dtype, device=proj.device)
         v_out = torch.empty(R, nv, dtype=torch.float32, device=proj.device) if want_v else None
         _hl().lig_qkv_norm_rope_cache(
-            _ptr(q_out), _ptr(v_out), _ptr(proj), proj.stride(0), _ptr(w_q) if mode else None,
-            _ptr(w_k) if mode else None, _ptr(inv_freq) if nf else None, nf, _ptr(positions),
+            _ptr(q_out), _ptr(v_out), _ptr(proj), proj.stride(0),
+            _ptr(w_q) if mode in (1, 2) else None, _ptr(w_k) if mode in (1, 2) else None, _ptr(inv_freq) if nf else None, nf, _ptr(positions),
             _ptr(v_first), float(lam), _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping),
             float(eps), R, heads, kv_heads, dim, vdim, mode, int(from_key),
-            int(bool(v_unit_norm)), bs, _is_f32(proj), _stream(),
+            int(bool(v_unit_norm)), bs, int(rot_layout == "interleaved"), _is_f32(proj),
+            _stream(),
         )
         return q_out, v_out
     return torch_ref.qkv_norm_rope_cache(
         proj, heads, kv_heads, dim, vdim, qk_norm, w_q, w_k, eps, inv_freq, positions,
         v_source, v_unit_norm, v_first, lam, want_v, k_cache, v_cache, slot_mapping,
+        rot_layout,
     )
 
 
@@ -1177,3 +1205,103 @@ def tanh_softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
         _hl().lig_tanh_softcap(_ptr(x), float(cap), x.numel(), _stream())
         return x
     return torch_ref.tanh_softcap(x, cap)
+
+
+# -- multi-stream residual, grouped router, routed combine ------------------------------
+
+def hyper_step(
+    xs: torch.Tensor, y: Optional[torch.Tensor], mix: Optional[torch.Tensor],
+    out_w: Optional[torch.Tensor], m: float, in_w: Optional[torch.Tensor],
+    g: Optional[torch.Tensor], eps: float, out_dtype,
+) -> Optional[torch.Tensor]:
+    """One step of a residual kept as S streams, xs fp32 [R, S, W], in place.
+
+    With y [R, W] (the output of the sub-layer that just ran): every stream
+    is rewritten from the old ones, x_t <- sum_s mix[s, t] x_s + m * out_w[t]
+    * y.  With in_w [S] (the next sub-layer's read): returns h = rms(u) * g
+    in out_dtype, u = sum_t in_w[t] x_t, g ONE fp32 weight (tensor of one
+    element).  mix, out_w, in_w, g are fp32 device tensors.  S == 1 with
+    unit coefficients is the plain pre-norm residual."""
+    assert xs.dtype == torch.float32 and xs.dim() == 3 and xs.is_contiguous()
+    R, S, W = xs.shape
+    if y is not None:
+        assert y.shape == (R, W) and y.is_contiguous() and y.dtype == out_dtype
+        assert mix.shape == (S, S) and out_w.shape == (S,)
+    if in_w is not None:
+        assert in_w.shape == (S,) and g.numel() == 1
+    if _use_hybrid(xs):
+        for t in (mix, out_w, in_w, g):
+            assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda)
+        h = torch.empty(R, W, dtype=out_dtype, device=xs.device) if in_w is not None else None
+        rc = _hl().lig_hyper_step(
+            _ptr(xs), _ptr(y), _ptr(mix), _ptr(out_w), float(m), _ptr(in_w), _ptr(g),
+            float(eps), _ptr(h), R, S, W, int(out_dtype == torch.float32), _stream(),
+        )
+        if rc != 0:
+            raise RuntimeError(f"hyper_step: {S} streams not served")
+        return h
+    return torch_ref.hyper_step(xs, y, mix, out_w, m, in_w, g, eps, out_dtype)
+
+
+def grouped_topk_route(
+    z: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int = 1,
+    keep: int = 1,
+):
+    """Softmax router with group-limited choice over fp32 logits z [T, N]:
+    scores s = softmax(z); choice scores s + correction; only outputs of the
+    `keep` groups (of N/groups neighbours) with the largest best choice score
+    can be chosen; the `top` largest choice scores win (ties: lower index).
+    Returns (idx int32 [T, top], weights fp32 [T, top] = chosen s over their
+    sum + 1e-20)."""
+    assert z.dtype == torch.float32 and z.dim() == 2 and z.is_contiguous()
+    T, N = z.shape
+    assert N % groups == 0 and 1 <= keep <= groups and 1 <= top <= keep * (N // groups)
+    if correction is not None:
+        assert correction.dtype == torch.float32 and correction.shape == (N,)
+    if _use_hybrid(z):
+        idx = torch.empty(T, top, dtype=torch.int32, device=z.device)
+        w = torch.empty(T, top, dtype=torch.float32, device=z.device)
+        rc = _hl().lig_grouped_topk_route(
+            _ptr(z), _ptr(correction), T, N, groups, keep, top, _ptr(idx), _ptr(w), _stream()
+        )
+        if rc != 0:
+            raise RuntimeError("grouped_topk_route: shape not served")
+        return idx, w
+    return torch_ref.grouped_topk_route(z, correction, top, groups, keep)
+
+
+def routed_combine(ye: torch.Tensor, x: torch.Tensor, rows: torch.Tensor, w: torch.Tensor):
+    """out[t] = sum_k w[t, k] * (ye[rows[t, k]] if rows[t, k] >= 0 else x[t]):
+    the weighted sum of a token's chosen expert outputs, a negative row
+    standing for an identity expert.  rows int64 [T, top], w fp32 [T, top]."""
+    T, W = x.shape
+    assert ye.dim() == 2 and ye.shape[1] == W and ye.dtype == x.dtype
+    assert rows.dtype == torch.int64 and w.dtype == torch.float32 and rows.shape == w.shape
+    if _use_hybrid(x):
+        assert ye.is_contiguous() and x.is_contiguous() and rows.is_contiguous() and w.is_contiguous()
+        out = torch.empty_like(x)
+        _hl().lig_routed_combine(
+            _ptr(out), _ptr(ye), _ptr(x), _ptr(rows), _ptr(w), T, rows.shape[1], W,
+            _is_f32(x), _stream(),
+        )
+        return out
+    return torch_ref.routed_combine(ye, x, rows, w)
+
+
+_GLU_KINDS = {"relu": 0, "clamped": 1}
+
+
+def glu_act(x: torch.Tensor, kind: str, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
+    """[rows, 2F] fused (gate | up) -> [rows, F].  "relu": relu(gate) * up.
+    "clamped": g = min(gate, limit), u = clamp(up, -limit, limit),
+    g * sigmoid(alpha * g) * (u + 1)."""
+    k = _GLU_KINDS[kind]
+    if _use_hybrid(x):
+        assert x.is_contiguous() and x.dim() == 2 and x.shape[1] % 2 == 0
+        F_ = x.shape[1] // 2
+        out = torch.empty(x.shape[0], F_, dtype=x.dtype, device=x.device)
+        _hl().lig_glu_act(
+            _ptr(out), _ptr(x), x.shape[0], F_, k, float(limit), float(alpha), _is_f32(x), _stream()
+        )
+        return out
+    return torch_ref.glu_act(x, kind, limit, alpha)

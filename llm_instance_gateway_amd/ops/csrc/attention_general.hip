@@ -23,6 +23,14 @@
 // floor(j / chunk) == floor(p / chunk), chunks counted from position 0 of the
 // sequence.
 //
+// window > 0 restricts a query at position p to keys j with p - j < window
+// (itself and the window - 1 tokens before it).
+//
+// sigmoid_weights: instead of a softmax every visible key weighs
+// sigmoid(score + score_bias[h]) (score_bias nullable, fp32 per head); the
+// weights are not normalised over the keys.  gate_per_head: the output gate
+// holds ONE entry per (token, head) instead of one per output element.
+//
 // Cache layout: K [blocks, G, BS, D], V [blocks, G, BS, v_row] of which the
 // first Dv entries of a row are the value (v_row == Dv for a cache of its
 // own; a latent cache passes the key rows themselves, v_row == D).
@@ -41,7 +49,8 @@ __global__ void paged_attention_general_kernel(
     const int64_t* __restrict__ positions,  // [R]
     const T* __restrict__ gate, long gate_stride, const float* __restrict__ sink,
     float scale, float temp_coef, float temp_every, int temp_every_int, int H,
-    int G, int D, int Dv, int v_row, int BS, int chunk) {
+    int G, int D, int Dv, int v_row, int BS, int chunk, int window,
+    const float* __restrict__ score_bias, int sigmoid_weights, int gate_per_head) {
   extern __shared__ __align__(16) float smem[];
   float* q_s = smem;                       // [D], padded to an even count
   float* p_s = smem + ((D + 1) & ~1);      // [64]
@@ -82,7 +91,9 @@ __global__ void paged_attention_general_kernel(
   for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) acc[i] = 0.f;
 
   // chunked visibility: the walk starts at the first key of the query's chunk
-  const int first_key = chunk > 0 ? (int)(pos / chunk) * chunk : 0;
+  int first_key = chunk > 0 ? (int)(pos / chunk) * chunk : 0;
+  if (window > 0) first_key = max(first_key, (int)pos - window + 1);
+  const float sb = score_bias != nullptr ? score_bias[h] : 0.f;
   for (int j0 = first_key; j0 < ctx; j0 += WAVE_SIZE) {
     const int j = j0 + lane;
     const bool valid = j < ctx;
@@ -106,11 +117,17 @@ __global__ void paged_attention_general_kernel(
       }
       score = dot * sc;
     }
-    const float m_new = fmaxf(m, wave_reduce_max(score));  // finite: key j0 is valid
-    const float p = valid ? expf(score - m_new) : 0.f;
-    const float alpha = expf(m - m_new);                   // 0 on the first tile
-    l = l * alpha + wave_reduce_sum(p);
-    m = m_new;
+    float p, alpha;
+    if (sigmoid_weights) {
+      p = valid ? sigmoid_f32(score + sb) : 0.f;
+      alpha = 1.f;
+    } else {
+      const float m_new = fmaxf(m, wave_reduce_max(score));  // finite: key j0 is valid
+      p = valid ? expf(score - m_new) : 0.f;
+      alpha = expf(m - m_new);                               // 0 on the first tile
+      l = l * alpha + wave_reduce_sum(p);
+      m = m_new;
+    }
     __syncthreads();  // previous tile's readers are done
     p_s[lane] = p;
     voff_s[lane] = voff;
@@ -126,13 +143,18 @@ __global__ void paged_attention_general_kernel(
       }
     }
   }
-  const float inv_l = 1.f / l;
+  const float inv_l = sigmoid_weights ? 1.f : 1.f / l;
+  float head_gate = 1.f;
+  if (gate != nullptr && gate_per_head)
+    head_gate = sigmoid_f32(ld(gate + (size_t)r * gate_stride + h));
 #pragma unroll
   for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
     const int d = lane + i * WAVE_SIZE;
     if (d < Dv) {
       float o = acc[i] * inv_l;
-      if (gate != nullptr)
+      if (gate_per_head)
+        o *= head_gate;
+      else if (gate != nullptr)
         o *= sigmoid_f32(ld(gate + (size_t)r * gate_stride + (size_t)h * Dv + d));
       st(orow + d, o);
     }
@@ -292,7 +314,8 @@ void lig_paged_attention_general(
     const int* tok_seq, const int64_t* positions, const void* gate,
     long gate_stride, const float* sink, float scale, float temp_coef,
     float temp_every, int temp_every_int, int R, int H, int G, int D, int Dv,
-    int v_row, int BS, int chunk, int is_f32, hipStream_t s) {
+    int v_row, int BS, int chunk, int window, const float* score_bias,
+    int sigmoid_weights, int gate_per_head, int is_f32, hipStream_t s) {
   if (R <= 0) return;
   dim3 grid(R, H), block(WAVE_SIZE);
   const size_t smem = (size_t)(((D + 1) & ~1) + WAVE_SIZE) * sizeof(float) + WAVE_SIZE * sizeof(long);
@@ -303,7 +326,8 @@ void lig_paged_attention_general(
                      (const T*)k_cache, (const T*)v_cache, block_tables,        \
                      max_blocks, tok_seq, positions, (const T*)gate,            \
                      gate_stride, sink, scale, temp_coef, temp_every,           \
-                     temp_every_int, H, G, D, Dv, v_row, BS, chunk)
+                     temp_every_int, H, G, D, Dv, v_row, BS, chunk, window,      \
+                     score_bias, sigmoid_weights, gate_per_head)
   if (is_f32) {
     if (vec) LIG_LAUNCH_ATT(float, true); else LIG_LAUNCH_ATT(float, false);
   } else {

@@ -19,7 +19,10 @@
 // length.  An optional per-head sink starts every row's running max at
 // sink_h and its running sum at one (a key with that unscaled score and no
 // value).  chunk > 0 restricts a row at position p to keys j with
-// floor(j / chunk) == floor(p / chunk).  A value row is the first Dv entries of a cache row of v_row
+// floor(j / chunk) == floor(p / chunk); window > 0 to keys j with
+// p - j < window.  sigmoid_weights replaces the softmax by unnormalised
+// weights sigmoid(score + score_bias[h]); gate_per_head reads one gate entry
+// per (row, head).  A value row is the first Dv entries of a cache row of v_row
 // entries, so a latent cache can pass its key rows as values.
 
 #include "elem_types.h"
@@ -43,7 +46,9 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
     const int* __restrict__ context_lens,      // [S] after this step's tokens
     const int* __restrict__ block_tables, float scale, float temp_coef,
     float temp_every, int temp_every_int, int num_q_heads, int num_kv_heads,
-    int D, int Dv, int v_row, int block_size, int max_blocks, int chunk) {
+    int D, int Dv, int v_row, int block_size, int max_blocks, int chunk,
+    int window, const float* __restrict__ score_bias, int sigmoid_weights,
+    int gate_per_head) {
   constexpr int DB = DVP / 16;
   constexpr int KB = DKP / 32;
 
@@ -114,8 +119,13 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
   // chunked visibility: a row at position p sees keys from floor(p / chunk)
   // * chunk on; the tile's walk starts at its first row's chunk
   const int qpos0 = ctx - n + qt;
-  const int kv_begin = chunk > 0 ? (qpos0 / chunk) * chunk : 0;
-  const int key_lo = (chunk > 0 && row_valid) ? (qpos / chunk) * chunk : 0;
+  int kv_begin = chunk > 0 ? (qpos0 / chunk) * chunk : 0;
+  int key_lo = (chunk > 0 && row_valid) ? (qpos / chunk) * chunk : 0;
+  if (window > 0) {
+    kv_begin = max(kv_begin, qpos0 - window + 1);
+    if (row_valid) key_lo = max(key_lo, qpos - window + 1);
+  }
+  const float sb = score_bias ? score_bias[h] : 0.f;
 
   for (int kv0 = kv_begin; kv0 < kv_end_tile; kv0 += PT_KVBLK) {
     // ---- staging: K rows [32][DKP], V transposed [DVP][32]; zero padding ----
@@ -188,7 +198,12 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
     float alpha;
     float psum = 0.0f;
     float p[8];
-    if (m_new == -INFINITY) {
+    if (sigmoid_weights) {
+      alpha = 1.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        p[i] = (sc[i] == -INFINITY) ? 0.0f : sigmoid_fast(sc[i] + sb);
+    } else if (m_new == -INFINITY) {
       alpha = 1.0f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) p[i] = 0.0f;
@@ -242,7 +257,7 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const float lr = __shfl(l, lg * 4 + r, 64);  // all lanes active here
-    inv_l[r] = lr > 0.f ? 1.0f / lr : 0.0f;
+    inv_l[r] = sigmoid_weights ? 1.0f : (lr > 0.f ? 1.0f / lr : 0.0f);
   }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -250,13 +265,18 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_tiles_kernel(
     if (orow >= n) continue;
     uint16_t* op = out + ((size_t)(lo + orow) * num_q_heads + h) * Dv;
     const uint16_t* gp =
-        gate ? gate + (size_t)(lo + orow) * gate_stride + (size_t)h * Dv : nullptr;
+        (gate && !gate_per_head)
+            ? gate + (size_t)(lo + orow) * gate_stride + (size_t)h * Dv : nullptr;
+    const float hg =
+        (gate && gate_per_head)
+            ? sigmoid_fast(bf16_to_f32(gate[(size_t)(lo + orow) * gate_stride + h])) : 1.0f;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
       const int d = db * 16 + li;
       if (d < Dv) {
         float o = acc_o[db][r] * inv_l[r];
         if (gp) o *= sigmoid_fast(bf16_to_f32(gp[d]));
+        o *= hg;
         op[d] = f32_to_bf16(o);
       }
     }
@@ -272,7 +292,8 @@ extern "C" int lig_paged_attention_prefill_tiles(
     const int* context_lens, const int* block_tables, float scale,
     float temp_coef, float temp_every, int temp_every_int, int ntiles,
     int num_q_heads, int num_kv_heads, int D, int Dv, int v_row, int block_size,
-    int max_blocks, int chunk, hipStream_t stream) {
+    int max_blocks, int chunk, int window, const float* score_bias,
+    int sigmoid_weights, int gate_per_head, hipStream_t stream) {
   if (D % 8 != 0 || Dv % 8 != 0 || D > 128 || Dv > 128 || D <= 0 || Dv <= 0 ||
       v_row % 8 != 0 || v_row < Dv ||
       q_stride % 8 != 0 || !aligned16(q) || !aligned16(k_cache) ||
@@ -290,7 +311,8 @@ extern "C" int lig_paged_attention_prefill_tiles(
                      query_start_locs,                                        \
                      context_lens, block_tables, scale, temp_coef, temp_every, \
                      temp_every_int, num_q_heads, num_kv_heads, D, Dv, v_row, \
-                     block_size, max_blocks, chunk)
+                     block_size, max_blocks, chunk, window, score_bias,       \
+                     sigmoid_weights, gate_per_head)
   const int dkp = D <= 32 ? 32 : (D <= 64 ? 64 : 128);
   const int dvp = Dv <= 32 ? 32 : (Dv <= 64 ? 64 : 128);
   if (dkp == 32 && dvp == 32) LAUNCH_PT(32, 32);

@@ -4,9 +4,11 @@
 //
 //   * q and k RMS norms: over the whole projection (weights of that size),
 //     per head (one weight of size D shared by the heads), or none;
-//   * rotate-half rotation of the first 2*n_freq entries of every q and k
-//     head: entry i pairs with entry i + n_freq, angle = float(pos) * f_i,
-//     accurate sincosf;
+//   * rotation of the first 2*n_freq entries of every q and k head, angle =
+//     float(pos) * f_i, accurate sincosf; rotate-half pairs entry i with
+//     entry i + n_freq, the interleaved layout pairs entry 2i with 2i + 1;
+//   * norm mode 3: q and k divided per head by their root mean square AFTER
+//     the rotation, without a weight;
 //   * values from their own columns or, v_from_key, the keys as projected
 //     (before the norm); optionally divided per head by their root mean
 //     square; optionally blended with another layer's values of the same
@@ -28,7 +30,8 @@ __global__ __launch_bounds__(256) void qkv_norm_rope_cache_kernel(
     const int64_t* __restrict__ positions, const float* __restrict__ v_first,
     float lam, T* __restrict__ k_cache, T* __restrict__ v_cache,
     const int64_t* __restrict__ slot_mapping, float eps, int H, int G, int D,
-    int Dv, int norm_mode, int v_from_key, int v_unit_norm, int BS) {
+    int Dv, int norm_mode, int v_from_key, int v_unit_norm, int BS,
+    int rot_interleaved) {
   extern __shared__ __align__(16) float sm[];
   __shared__ float red[17];
   const int nq = H * D, nk = G * D, nv = G * Dv;
@@ -110,9 +113,22 @@ __global__ __launch_bounds__(256) void qkv_norm_rope_cache_kernel(
       float* v = hh < H ? q_s + hh * D : k_s + (hh - H) * D;
       float sn, cs;
       sincosf(fp * inv_freq[i], &sn, &cs);
-      const float a = v[i], b = v[i + n_freq];
-      v[i] = a * cs - b * sn;
-      v[i + n_freq] = b * cs + a * sn;
+      const int ia = rot_interleaved ? 2 * i : i;
+      const int ib = rot_interleaved ? 2 * i + 1 : i + n_freq;
+      const float a = v[ia], b = v[ib];
+      v[ia] = a * cs - b * sn;
+      v[ib] = b * cs + a * sn;
+    }
+    __syncthreads();
+  }
+  if (norm_mode == 3) {
+    for (int hh = wave; hh < H + G; hh += nwaves) {
+      float* v = hh < H ? q_s + hh * D : k_s + (hh - H) * D;
+      float ss = 0.f;
+      for (int d = lane; d < D; d += WAVE_SIZE) ss += v[d] * v[d];
+      ss = wave_reduce_sum(ss);
+      const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+      for (int d = lane; d < D; d += WAVE_SIZE) v[d] *= inv;
     }
     __syncthreads();
   }
@@ -162,8 +178,8 @@ extern "C" void lig_qkv_norm_rope_cache(
     const void* w_k, const float* inv_freq, int n_freq, const int64_t* positions,
     const float* v_first, float lam, void* k_cache, void* v_cache,
     const int64_t* slot_mapping, float eps, int R, int H, int G, int D, int Dv,
-    int norm_mode, int v_from_key, int v_unit_norm, int BS, int is_f32,
-    hipStream_t s) {
+    int norm_mode, int v_from_key, int v_unit_norm, int BS, int rot_interleaved,
+    int is_f32, hipStream_t s) {
   if (R <= 0) return;
   const size_t smem = (size_t)(H * D + G * D + G * Dv) * sizeof(float);
   const bool vec = D % 8 == 0 && Dv % 8 == 0 && proj_stride % 8 == 0 && aligned16(proj) &&
@@ -173,7 +189,7 @@ extern "C" void lig_qkv_norm_rope_cache(
                      s, (T*)q_out, v_out, (const T*)proj, proj_stride,              \
                      (const T*)w_q, (const T*)w_k, inv_freq, n_freq, positions,     \
                      v_first, lam, (T*)k_cache, (T*)v_cache, slot_mapping, eps, H,  \
-                     G, D, Dv, norm_mode, v_from_key, v_unit_norm, BS)
+                     G, D, Dv, norm_mode, v_from_key, v_unit_norm, BS, rot_interleaved)
   if (is_f32) {
     if (vec) LIG_QP(float, true); else LIG_QP(float, false);
   } else {

@@ -1,6 +1,7 @@
 """Light native library for the hybrid-model kernels (grouped RMS norm, xIELU,
 minGRU scan, general-size paged attention, shift norms, latent attention,
-sum+norm residual step, q/k/v prep, head-mixed attention, matrix-state scan).
+sum+norm residual step, q/k/v prep, head-mixed attention, matrix-state scan,
+multi-stream residual step, grouped router and routed combine).
 
 These kernels expose a plain C ABI and need no torch headers, so they are
 compiled by one direct ``hipcc -shared`` call (seconds, not the minutes the
@@ -33,7 +34,8 @@ SOURCES = [
     "group_norm.hip", "xielu.hip", "mingru.hip", "attention_general.hip",
     "attention_prefill_tiles.hip", "shift_norm.hip", "latent_attention.hip", "ff_act.hip",
     "attention_latent_rows.hip", "post_norm.hip", "qkv_prep.hip", "attention_mixed_heads.hip",
-    "matrix_state_scan.hip", "attention_mixed_heads_tiles.hip",
+    "matrix_state_scan.hip", "attention_mixed_heads_tiles.hip", "hyper_streams.hip",
+    "routed.hip",
 ]
 SO_PATH = PKG / "_hybrid.so"
 
@@ -81,7 +83,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "lig_sigmoid_gate_mul": [p, p, l, i, i, i, p],
         "lig_mingru_scan": [p, p, p, p, l, p, p, p, p, p, p, i, i, i, i, p],
         "lig_paged_attention_general": [
-            p, p, l, p, p, p, i, p, p, p, l, p, f, f, f, i, i, i, i, i, i, i, i, i, i, p,
+            p, p, l, p, p, p, i, p, p, p, l, p, f, f, f, i, i, i, i, i, i, i, i, i,
+            i, p, i, i, i, p,
         ],
         "lig_offset_norm_shift": [p, p, p, p, p, p, p, p, p, p, p, p, p, p, p, f, i, i, i, p],
         "lig_offset_rms_norm": [p, p, p, f, i, i, i, p],
@@ -95,21 +98,32 @@ def _declare(lib: ctypes.CDLL) -> None:
         "lig_temperature_scale_rows": [p, p, l, p, f, f, i, i, i, i, p],
         "lig_scaled_add_rms_norm": [p, p, p, p, p, f, f, f, f, i, i, i, p],
         "lig_qkv_norm_rope_cache": [
-            p, p, p, l, p, p, p, i, p, p, f, p, p, p, f, i, i, i, i, i, i, i, i, i, i, p,
+            p, p, p, l, p, p, p, i, p, p, f, p, p, p, f, i, i, i, i, i, i, i, i, i, i, i, p,
         ],
         "lig_token_shift_mix": [p, p, p, p, p, p, p, p, p, i, i, i, i, p],
         "lig_group_rms_norm_gate": [p, p, p, l, p, i, i, f, i, i, i, p],
         "lig_gelu_erf": [p, p, l, i, p],
         "lig_tanh_act": [p, p, l, i, p],
         "lig_tanh_softcap": [p, f, l, p],
+        "lig_routed_combine": [p, p, p, p, p, i, i, i, i, p],
+        "lig_glu_act": [p, p, l, i, i, f, f, i, p],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = None
     pt = lib.lig_paged_attention_prefill_tiles
-    pt.argtypes = [p, p, l, p, p, p, l, p, p, p, p, p, p, f, f, f, i, i, i, i, i, i, i, i, i, i, p]
+    pt.argtypes = [
+        p, p, l, p, p, p, l, p, p, p, p, p, p, f, f, f, i, i, i, i, i, i, i, i, i, i,
+        i, p, i, i, p,
+    ]
     pt.restype = ctypes.c_int
+    hs = lib.lig_hyper_step
+    hs.argtypes = [p, p, p, p, f, p, p, f, p, i, i, i, i, p]
+    hs.restype = ctypes.c_int
+    gr = lib.lig_grouped_topk_route
+    gr.argtypes = [p, p, i, i, i, i, i, p, p, p]
+    gr.restype = ctypes.c_int
     mh = lib.lig_paged_attention_mixed_heads
     mh.argtypes = [p, p, l, p, p, p, i, p, p, p, i, p, f, i, i, i, i, i, i, i, i, p]
     mh.restype = ctypes.c_int

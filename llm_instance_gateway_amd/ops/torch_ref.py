@@ -291,14 +291,18 @@ def query_temperature(positions: torch.Tensor, coef: float, every: float) -> tor
 def paged_attention_general(
     q, k_cache, v_cache, block_tables, tok_seq, positions, scale: float,
     num_heads: int, gate=None, temp_coef: float = 0.0, temp_every: float = 1.0,
-    sink=None, chunk: int = 0,
+    sink=None, chunk: int = 0, window: int = 0, score_bias=None,
+    weights: str = "softmax", gate_per_head: bool = False,
 ):
     """q [R, H*D] (may be a strided view); token r belongs to sequence row
     tok_seq[r] of block_tables (-1: padding row) and sees keys 0..positions[r].
     `sink` [H] fp32 adds exp(sink_h) to head h's softmax denominator (a key
     with that unscaled score and no value).  v_cache may be a view into
     k_cache's rows.  chunk > 0 hides keys of earlier chunks: key j is seen
-    only if floor(j / chunk) == floor(position / chunk)."""
+    only if floor(j / chunk) == floor(position / chunk); window > 0 hides
+    keys with position - j >= window.  weights "sigmoid": unnormalised
+    sigmoid(score + score_bias[h]) per visible key.  gate_per_head: gate
+    [R, H]."""
     R = q.shape[0]
     nb, G, bs, D = k_cache.shape
     Dv = v_cache.shape[-1]
@@ -331,14 +335,22 @@ def paged_attention_general(
             mask = keyp > positions[r:e, None]
             if chunk > 0:
                 mask = mask | (keyp < (positions[r:e, None] // chunk) * chunk)
+            if window > 0:
+                mask = mask | (keyp < positions[r:e, None] - window + 1)
             sc.masked_fill_(mask[None], float("-inf"))
-            if sink is not None:
+            if weights == "sigmoid":
+                if score_bias is not None:
+                    sc = sc + score_bias.float().view(H, 1, 1)
+                pr = torch.sigmoid(sc)  # sigmoid(-inf) = 0
+            elif sink is not None:
                 sk = sink.float().view(H, 1, 1).expand(H, e - r, 1)
                 pr = torch.softmax(torch.cat([sc, sk], dim=-1), dim=-1)[..., :-1]
             else:
                 pr = torch.softmax(sc, dim=-1)
             o = torch.bmm(pr, vf).permute(1, 0, 2).reshape(e - r, H * Dv)
-            if gate is not None:
+            if gate is not None and gate_per_head:
+                o = (o.view(e - r, H, Dv) * torch.sigmoid(gate[r:e].float())[:, :, None]).reshape(e - r, H * Dv)
+            elif gate is not None:
                 o = o * torch.sigmoid(gate[r:e].float())
             out[r:e] = o.to(out.dtype)
         r = e
@@ -399,10 +411,12 @@ def offset_norm_shift(
     return hm.to(out_dtype), hf
 
 
-def rotary_inv_freq(base: float, dims: int, device=None) -> torch.Tensor:
-    """f_i = base^(-2i/dims), i < dims/2, evaluated in float64, stored fp32."""
+def rotary_inv_freq(base: float, dims: int, device=None, divide: float = 1.0) -> torch.Tensor:
+    """f_i = base^(-2i/dims) / divide, i < dims/2, evaluated in float64, stored
+    fp32 (divide > 1 is linear position scaling)."""
     i = torch.arange(dims // 2, dtype=torch.float64)
-    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float().to(device)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims) / float(divide)
+    return f.float().to(device)
 
 
 def _rotate_pairs(v: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
@@ -495,7 +509,7 @@ def _rotate_halves(v: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Ten
 def qkv_norm_rope_cache(
     proj, heads: int, kv_heads: int, dim: int, vdim: int, qk_norm: str, w_q, w_k,
     eps: float, inv_freq, positions, v_source: str, v_unit_norm: bool, v_first,
-    lam: float, want_v: bool, k_cache, v_cache, slot_mapping,
+    lam: float, want_v: bool, k_cache, v_cache, slot_mapping, rot_layout: str = "half",
 ):
     R = proj.shape[0]
     nq, nk = heads * dim, kv_heads * dim
@@ -513,8 +527,11 @@ def qkv_norm_rope_cache(
     else:
         q, k = q.reshape(R, heads, dim), k.reshape(R, kv_heads, dim)
     if inv_freq is not None and inv_freq.numel() > 0:
-        q = _rotate_halves(q, positions, inv_freq)
-        k = _rotate_halves(k, positions, inv_freq)
+        rot = _rotate_halves if rot_layout == "half" else _rotate_pairs
+        q = rot(q, positions, inv_freq)
+        k = rot(k, positions, inv_freq)
+    if qk_norm == "head_post":
+        q, k = _rms_scale(q, eps), _rms_scale(k, eps)
     if v_unit_norm:
         v = _rms_scale(v, eps)
     if v_first is not None:
@@ -641,3 +658,48 @@ def tanh_act(x: torch.Tensor) -> torch.Tensor:
 
 def tanh_softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
     return x.copy_(cap * torch.tanh(x.float() / cap))
+
+
+def hyper_step(xs, y, mix, out_w, m: float, in_w, g, eps: float, out_dtype):
+    """xs fp32 [R, S, W] in place: with y, x_t <- sum_s mix[s, t] x_s + m *
+    out_w[t] * y; with in_w, returns rms(sum_t in_w[t] x_t) * g."""
+    if y is not None:
+        new = torch.einsum("st,rsw->rtw", mix.float(), xs) + (m * out_w.float())[None, :, None] * y.float()[:, None, :]
+        xs.copy_(new)
+    if in_w is None:
+        return None
+    u = torch.einsum("s,rsw->rw", in_w.float(), xs)
+    return (_rms_scale(u, eps) * g.float().reshape(())).to(out_dtype)
+
+
+def grouped_topk_route(z, correction, top: int, groups: int, keep: int):
+    T, N = z.shape
+    s = torch.softmax(z.float(), dim=-1)
+    c = s if correction is None else s + correction.float()[None, :]
+    if groups > 1 and keep < groups:
+        per = N // groups
+        gs = c.view(T, groups, per).max(dim=-1).values
+        # stable order: ties go to the lower index
+        order = torch.argsort(-gs, dim=-1, stable=True)[:, :keep]
+        allowed = torch.zeros(T, groups, dtype=torch.bool, device=z.device).scatter_(1, order, True)
+        c = c.masked_fill(~allowed.repeat_interleave(per, dim=1), float("-inf"))
+    idx = torch.argsort(-c, dim=-1, stable=True)[:, :top]
+    w = s.gather(1, idx)
+    return idx.to(torch.int32), w / (w.sum(dim=-1, keepdim=True) + 1e-20)
+
+
+def routed_combine(ye, x, rows, w):
+    T, W = x.shape
+    src = torch.cat([ye, x], dim=0).float()
+    at = torch.where(rows >= 0, rows, ye.shape[0] + torch.arange(T, device=x.device)[:, None])
+    return (src[at] * w[:, :, None]).sum(dim=1).to(x.dtype)
+
+
+def glu_act(x, kind: str, limit: float, alpha: float):
+    F_ = x.shape[1] // 2
+    g, u = x[:, :F_].float(), x[:, F_:].float()
+    if kind == "relu":
+        return (torch.relu(g) * u).to(x.dtype)
+    g = g.clamp(max=limit)
+    u = u.clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(x.dtype)
