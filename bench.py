@@ -132,7 +132,27 @@ def main() -> None:
         "both (benchmarks/bench_postnorm.py)",
     )
     ap.add_argument("--postnorm-sizes", default="s,m")
+    ap.add_argument(
+        "--streams",
+        nargs="?",
+        const="engine,kernels",
+        default="",
+        metavar="PARTS",
+        help="instead of the serving workload: Vemenex (multi-stream "
+        "residual, sliding-window sigmoid / sink attention, group-routed "
+        "experts) beside Potatar's attention layers and Mixtral at equal "
+        "size, and its kernels beside their counterparts against the "
+        "roofline; PARTS = engine, kernels or both (benchmarks/bench_streams.py)",
+    )
+    ap.add_argument("--streams-sizes", default="s,m")
     args = ap.parse_args()
+
+    if args.streams:
+        sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmarks"))
+        import bench_streams
+
+        bench_streams.main(["--part", args.streams, "--sizes", args.streams_sizes])
+        return
 
     if args.postnorm:
         sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmarks"))
