@@ -13,11 +13,15 @@ feed-forward.  The routed variant stands beside Mixtral with the same
 experts.
 
 Engine part: for each size a dense Vemenex stack (sigmoid-weight and
-sink-softmax attention alternating, window 512, two residual streams, gated
-relu feed-forward) beside a Potatar stack of chunk-512 attention layers with
-the same width, depth, heads and feed-forward parameters; and a routed
-Vemenex stack (8 experts + 2 identity experts in 2 groups of which 1 is
-kept, 2 per token, in every layer) beside Mixtral (8 experts, 2 per token).
+sink-softmax attention alternating, two residual streams, gated relu
+feed-forward) beside a Potatar stack of attention layers with the same
+width, depth, heads and feed-forward parameters; and a routed Vemenex stack
+(8 experts + 2 identity experts in 2 groups of which 1 is kept, 2 per token,
+in every layer) beside Mixtral (8 experts, 2 per token).  A sliding window
+and a chunk of the same size see different numbers of keys (a chunk starts
+anew every `size` positions), so here both masks are as long as the longest
+sequence of the workload and every query sees its whole past, as in Mixtral;
+the kernel part times both masks at 512 with equal numbers of visible keys.
 The same workload goes through LLMEngine.step(): N prompts of L tokens in
 budget-sized steps, then K decode steps (hipGraph replay) at batch N.
 Random weights, synthetic tokens.
@@ -56,7 +60,7 @@ WINDOW = 512
 EXPERTS, IDENTITY, TOP = 8, 2, 2
 
 
-def vemenex_config(name: str, z: dict, routed: bool) -> ModelConfig:
+def vemenex_config(name: str, z: dict, routed: bool, mask: int = WINDOW) -> ModelConfig:
     layers = []
     for i in range(z["layers"]):
         kind = "attention" if i % 2 == 0 else "attention_2"
@@ -72,20 +76,20 @@ def vemenex_config(name: str, z: dict, routed: bool) -> ModelConfig:
         layers.append({
             "type": kind,
             "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
-                      "mask": {"size": WINDOW}, "rot": rot, "scale": 1.0 / math.sqrt(z["dim"])},
+                      "mask": {"size": mask}, "rot": rot, "scale": 1.0 / math.sqrt(z["dim"])},
             "mlp": mlp,
         })
     return make_config(f"vemenex-{name}{'-routed' if routed else ''}", z["vocab"], z["width"], layers,
                        eps=1e-6, residual_mult=0.5, streams=2)
 
 
-def potatar_attention_config(name: str, z: dict) -> ModelConfig:
+def potatar_attention_config(name: str, z: dict, mask: int = WINDOW) -> ModelConfig:
     """Attention layers only; the two-matrix feed-forward is widened to the
     parameter count of the three-matrix one."""
     att = {
         "type": "attention",
         "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
-                  "mask": {"size": WINDOW}, "rot": {"base": 10000.0, "dims": z["dim"] // 2},
+                  "mask": {"size": mask}, "rot": {"base": 10000.0, "dims": z["dim"] // 2},
                   "scale": 1.0 / math.sqrt(z["dim"]), "v_mix": False},
         "mlp": {"ff": z["ff"] * 3 // 2, "kind": "dense"},
     }
@@ -106,11 +110,13 @@ def part_engine(sizes) -> None:
     for name in sizes:
         z = SIZES[name]
         for n_seqs, plen in ((16, 1024), (64, 512)):
-            row = {"bench": "engine", "size": name, **z, "seqs": n_seqs, "prompt_len": plen, "decode_steps": 64}
-            row["vemenex_dense"] = engine_run(vemenex_config(name, z, False), n_seqs, plen, 64)
-            row["potatar_attention"] = engine_run(potatar_attention_config(name, z), n_seqs, plen, 64)
+            mask = plen + 64 + 1
+            row = {"bench": "engine", "size": name, **z, "seqs": n_seqs, "prompt_len": plen, "decode_steps": 64,
+                   "mask": mask}
+            row["vemenex_dense"] = engine_run(vemenex_config(name, z, False, mask), n_seqs, plen, 64)
+            row["potatar_attention"] = engine_run(potatar_attention_config(name, z, mask), n_seqs, plen, 64)
             if plen == 1024:
-                row["vemenex_routed"] = engine_run(vemenex_config(name, z, True), n_seqs, plen, 64)
+                row["vemenex_routed"] = engine_run(vemenex_config(name, z, True, mask), n_seqs, plen, 64)
                 row["mixtral"] = engine_run(mixtral_config(name, z), n_seqs, plen, 64)
             for k in ("prefill_tok_per_s", "decode_tok_per_s"):
                 row["dense_vs_potatar_" + k] = round(row["vemenex_dense"][k] / row["potatar_attention"][k], 3)

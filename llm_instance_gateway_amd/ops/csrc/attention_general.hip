@@ -39,8 +39,14 @@
 
 #define ATT_MAX_DV_PER_LANE 8  // Dv <= 512
 
-template <typename T, bool VEC>
-__global__ void paged_attention_general_kernel(
+// NW waves of a workgroup share one (token, head): wave w takes the 64-key
+// tiles w, w + NW, ... of the walk and keeps its own running max / sum /
+// accumulator; wave 0 merges them through LDS at the end.  Small batches of
+// single tokens, which would otherwise leave most of the chip idle behind one
+// serial walk per wave, run with NW = 4.  Every wave makes the same number of
+// loop trips (a trip without a tile only meets the barriers).
+template <typename T, bool VEC, int NW>
+__global__ __launch_bounds__(WAVE_SIZE * NW) void paged_attention_general_kernel(
     T* __restrict__ out,  // [R, H * Dv]
     const T* __restrict__ q, long q_stride,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -52,15 +58,21 @@ __global__ void paged_attention_general_kernel(
     int G, int D, int Dv, int v_row, int BS, int chunk, int window,
     const float* __restrict__ score_bias, int sigmoid_weights, int gate_per_head) {
   extern __shared__ __align__(16) float smem[];
-  float* q_s = smem;                       // [D], padded to an even count
-  float* p_s = smem + ((D + 1) & ~1);      // [64]
-  long* voff_s = reinterpret_cast<long*>(p_s + WAVE_SIZE);  // [64]
+  const int Dpad = (D + 1) & ~1;
+  float* q_s = smem;                                   // [D], padded to an even count
+  float* p_all = smem + Dpad;                          // [NW][64]
+  long* voff_all = reinterpret_cast<long*>(p_all + NW * WAVE_SIZE);  // [NW][64]
+  float* ml_s = reinterpret_cast<float*>(voff_all + NW * WAVE_SIZE);  // [NW][2]
+  float* acc_s = ml_s + 2 * NW;                        // [NW][Dv]
 
-  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int r = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x % WAVE_SIZE, wave = threadIdx.x / WAVE_SIZE;
+  float* p_s = p_all + wave * WAVE_SIZE;
+  long* voff_s = voff_all + wave * WAVE_SIZE;
   const int seq = tok_seq[r];
   T* orow = out + (size_t)r * H * Dv + (size_t)h * Dv;
   if (seq < 0) {
-    for (int d = lane; d < Dv; d += WAVE_SIZE) st(orow + d, 0.f);
+    for (int d = threadIdx.x; d < Dv; d += WAVE_SIZE * NW) st(orow + d, 0.f);
     return;
   }
   const long pos = positions[r];
@@ -78,11 +90,11 @@ __global__ void paged_attention_general_kernel(
   const float sc = scale * tau;
 
   const T* qrow = q + (size_t)r * q_stride + (size_t)h * D;
-  for (int d = lane; d < D; d += WAVE_SIZE) q_s[d] = ld(qrow + d);
+  for (int d = threadIdx.x; d < D; d += WAVE_SIZE * NW) q_s[d] = ld(qrow + d);
   __syncthreads();
 
   float m = -INFINITY, l = 0.f;
-  if (sink != nullptr) {
+  if (sink != nullptr && wave == 0) {  // the sink is counted once
     m = sink[h];
     l = 1.f;
   }
@@ -94,9 +106,14 @@ __global__ void paged_attention_general_kernel(
   int first_key = chunk > 0 ? (int)(pos / chunk) * chunk : 0;
   if (window > 0) first_key = max(first_key, (int)pos - window + 1);
   const float sb = score_bias != nullptr ? score_bias[h] : 0.f;
-  for (int j0 = first_key; j0 < ctx; j0 += WAVE_SIZE) {
+  const int ntiles = (ctx - first_key + WAVE_SIZE - 1) / WAVE_SIZE;
+  const int trips = (ntiles + NW - 1) / NW;
+  for (int it = 0; it < trips; ++it) {
+    const int tile = it * NW + wave;
+    const bool active = tile < ntiles;  // uniform over the wave
+    const int j0 = first_key + tile * WAVE_SIZE;
     const int j = j0 + lane;
-    const bool valid = j < ctx;
+    const bool valid = active && j < ctx;
     float score = -INFINITY;
     long voff = 0;
     if (valid) {
@@ -117,29 +134,70 @@ __global__ void paged_attention_general_kernel(
       }
       score = dot * sc;
     }
-    float p, alpha;
-    if (sigmoid_weights) {
-      p = valid ? sigmoid_f32(score + sb) : 0.f;
-      alpha = 1.f;
-    } else {
-      const float m_new = fmaxf(m, wave_reduce_max(score));  // finite: key j0 is valid
-      p = valid ? expf(score - m_new) : 0.f;
-      alpha = expf(m - m_new);                               // 0 on the first tile
-      l = l * alpha + wave_reduce_sum(p);
-      m = m_new;
+    float p = 0.f, alpha = 1.f;
+    if (active) {
+      if (sigmoid_weights) {
+        p = valid ? sigmoid_f32(score + sb) : 0.f;
+      } else {
+        const float m_new = fmaxf(m, wave_reduce_max(score));  // finite: key j0 is valid
+        p = valid ? expf(score - m_new) : 0.f;
+        alpha = expf(m - m_new);                               // 0 on the wave's first tile
+        l = l * alpha + wave_reduce_sum(p);
+        m = m_new;
+      }
     }
     __syncthreads();  // previous tile's readers are done
     p_s[lane] = p;
     voff_s[lane] = voff;
     __syncthreads();
-    const int nv = min(WAVE_SIZE, ctx - j0);
+    if (active) {
+      const int nv = min(WAVE_SIZE, ctx - j0);
+#pragma unroll
+      for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
+        const int d = lane + i * WAVE_SIZE;
+        if (d < Dv) {
+          float a = acc[i] * alpha;
+          for (int jj = 0; jj < nv; ++jj) a += p_s[jj] * ld(v_cache + voff_s[jj] + d);
+          acc[i] = a;
+        }
+      }
+    }
+  }
+  if (NW > 1) {
+    // wave 0 gathers the other waves' partial results
+    if (lane == 0) {
+      ml_s[2 * wave] = m;
+      ml_s[2 * wave + 1] = l;
+    }
 #pragma unroll
     for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
       const int d = lane + i * WAVE_SIZE;
-      if (d < Dv) {
-        float a = acc[i] * alpha;
-        for (int jj = 0; jj < nv; ++jj) a += p_s[jj] * ld(v_cache + voff_s[jj] + d);
-        acc[i] = a;
+      if (d < Dv) acc_s[wave * Dv + d] = acc[i];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    if (sigmoid_weights) {
+#pragma unroll
+      for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
+        const int d = lane + i * WAVE_SIZE;
+        if (d < Dv)
+          for (int w = 1; w < NW; ++w) acc[i] += acc_s[w * Dv + d];
+      }
+    } else {
+      float M = m;  // finite: wave 0 always has the walk's first key
+      for (int w = 1; w < NW; ++w) M = fmaxf(M, ml_s[2 * w]);
+      const float f0 = expf(m - M);
+      l *= f0;
+#pragma unroll
+      for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) acc[i] *= f0;
+      for (int w = 1; w < NW; ++w) {
+        const float fw = expf(ml_s[2 * w] - M);  // 0 for a wave without tiles
+        l += ml_s[2 * w + 1] * fw;
+#pragma unroll
+        for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
+          const int d = lane + i * WAVE_SIZE;
+          if (d < Dv) acc[i] += acc_s[w * Dv + d] * fw;
+        }
       }
     }
   }
@@ -317,22 +375,29 @@ void lig_paged_attention_general(
     int v_row, int BS, int chunk, int window, const float* score_bias,
     int sigmoid_weights, int gate_per_head, int is_f32, hipStream_t s) {
   if (R <= 0) return;
-  dim3 grid(R, H), block(WAVE_SIZE);
-  const size_t smem = (size_t)(((D + 1) & ~1) + WAVE_SIZE) * sizeof(float) + WAVE_SIZE * sizeof(long);
+  // few rows: four waves share each (token, head) so the walk is split
+  const int nw = (long)R * H <= 4096 ? 4 : 1;
+  dim3 grid(R, H), block(WAVE_SIZE * nw);
+  const size_t smem = (size_t)(((D + 1) & ~1) + nw * WAVE_SIZE) * sizeof(float) +
+                      (size_t)nw * WAVE_SIZE * sizeof(long) +
+                      (size_t)nw * (2 + Dv) * sizeof(float);
   const bool vec = D % 8 == 0 && aligned16(k_cache);
-#define LIG_LAUNCH_ATT(T, VEC)                                                  \
-  hipLaunchKernelGGL((paged_attention_general_kernel<T, VEC>), grid, block,     \
+#define LIG_LAUNCH_ATT(T, VEC, NW)                                              \
+  hipLaunchKernelGGL((paged_attention_general_kernel<T, VEC, NW>), grid, block, \
                      smem, s, (T*)out, (const T*)q, q_stride,                   \
                      (const T*)k_cache, (const T*)v_cache, block_tables,        \
                      max_blocks, tok_seq, positions, (const T*)gate,            \
                      gate_stride, sink, scale, temp_coef, temp_every,           \
                      temp_every_int, H, G, D, Dv, v_row, BS, chunk, window,      \
                      score_bias, sigmoid_weights, gate_per_head)
+#define LIG_LAUNCH_ATT_W(T, VEC) \
+  if (nw == 4) LIG_LAUNCH_ATT(T, VEC, 4); else LIG_LAUNCH_ATT(T, VEC, 1)
   if (is_f32) {
-    if (vec) LIG_LAUNCH_ATT(float, true); else LIG_LAUNCH_ATT(float, false);
+    if (vec) { LIG_LAUNCH_ATT_W(float, true); } else { LIG_LAUNCH_ATT_W(float, false); }
   } else {
-    if (vec) LIG_LAUNCH_ATT(bf16s, true); else LIG_LAUNCH_ATT(bf16s, false);
+    if (vec) { LIG_LAUNCH_ATT_W(bf16s, true); } else { LIG_LAUNCH_ATT_W(bf16s, false); }
   }
+#undef LIG_LAUNCH_ATT_W
 #undef LIG_LAUNCH_ATT
 }
 
