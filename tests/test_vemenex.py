@@ -64,7 +64,7 @@ CFG_A = {
 # window of one token, a window longer than any prompt, a rotation that
 # leaves most of the head alone, one expert, every output in one group
 CFG_B = {
-    "architecture": "Vemenex", "vocab": 61, "width": 24, "norm": {"eps": 1e-6},
+    "architecture": "Vemenex", "vocab": 61, "width": 26, "norm": {"eps": 1e-6},
     "residual_mult": 1.0, "streams": 1,
     "layers": [
         att("attention", 1, 1, 6, 3, 1, 2, moe(7, 1, 1)),
@@ -84,6 +84,19 @@ CFG_C = {
         att("attention_2", 2, 1, 64, 64, 128, 32, moe(16, 4, 2, identity=2, groups=3, keep=2)),
         att("attention", 4, 2, 24, 16, 33, 24, None),
         att("attention_2", 4, 2, 16, 40, 64, 8, dense(48)),
+    ],
+}
+
+
+# no routed layer anywhere (the runner then pads the flat batch for the
+# GEMMs, so rows of no sequence pass through every kernel), two streams
+CFG_D = {
+    "architecture": "Vemenex", "vocab": 70, "width": 32, "norm": {"eps": 1e-5},
+    "residual_mult": 1.3, "streams": 2,
+    "layers": [
+        att("attention_2", 4, 1, 8, 8, 9, 8, dense(40)),
+        att("attention", 2, 2, 16, 8, 25, 8, None, factor=8.0),
+        att("attention", 3, 1, 8, 16, 40, 4, dense(16)),
     ],
 }
 
@@ -226,6 +239,11 @@ def model_c(tmp_path_factory):
 
 
 @pytest.fixture(scope="module")
+def model_d(tmp_path_factory):
+    return _model(tmp_path_factory, CFG_D, 34, "d")
+
+
+@pytest.fixture(scope="module")
 def oracle_a(model_a):
     toks = tokens_for(CFG_A, 90, 5)
     return (toks,) + oracle(CFG_A, model_a[1], toks)
@@ -265,13 +283,16 @@ def test_whole_prompt_and_every_layer(model_a, oracle_a, device, dtype):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("which", ["b", "c"])
-def test_other_sizes(model_b, model_c, device, which):
-    cfg, (path, W) = (CFG_B, model_b) if which == "b" else (CFG_C, model_c)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["b", "c", "d"])
+def test_other_sizes(model_b, model_c, model_d, device, dtype, which):
+    if device == "cpu" and dtype == torch.bfloat16:
+        pytest.skip("bf16 is the GPU serving precision")
+    cfg, (path, W) = {"b": (CFG_B, model_b), "c": (CFG_C, model_c), "d": (CFG_D, model_d)}[which]
     toks = tokens_for(cfg, 75, 6)
     want, _ = oracle(cfg, W, toks)
-    eng = make_engine(path, device, block_size=8)
-    assert_logits(replay_all(eng, "d", toks, [17, 1, 1, 2, 19, 35]), want)
+    eng = make_engine(path, device, dtype, block_size=8)
+    assert_logits(replay_all(eng, "d", toks, [17, 1, 1, 2, 19, 35]), want, dtype)
 
 
 @pytest.mark.parametrize("device", DEVICES)
