@@ -906,7 +906,7 @@ class GroupRoutedExpertsMLP(nn.Module):
     def route(self, h: torch.Tensor):
         z = F.linear(h.float(), self.w_router)
         idx, w = ops.grouped_topk_route(z, self.correction, self.top, self.groups, self.keep)
-        return w, idx.long()
+        return w, idx  # fp32 [T, top], int32 [T, top]
 
     def _experts(self, xe: torch.Tensor, rows: int) -> torch.Tensor:
         """xe [E, rows, hidden] -> [E * rows, hidden]."""
@@ -920,10 +920,8 @@ class GroupRoutedExpertsMLP(nn.Module):
         w, idx = self.route(h)
         if meta is not None and meta.num_prefill_tokens == 0:
             ye = self._experts(h.unsqueeze(0).expand(E, T, hidden), T)
-            tok = torch.arange(T, device=h.device).unsqueeze(1)
-            rows = torch.where(idx < E, idx * T + tok, torch.full_like(idx, -1))
-            return ops.routed_combine(ye, h, rows.contiguous(), w)
-        gather, rows, cap = expert_dispatch_plan(idx, E)
+            return ops.routed_combine(ye, h, None, w, idx=idx, experts=E)
+        gather, rows, cap = expert_dispatch_plan(idx.long(), E)
         xe = ops.scale_gather_rows(h, gather, (gather >= 0).float())
         ye = self._experts(xe.view(E, cap, hidden), cap)
         return ops.routed_combine(ye, h, rows.contiguous(), w)

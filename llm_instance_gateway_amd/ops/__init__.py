@@ -1270,21 +1270,37 @@ def grouped_topk_route(
     return torch_ref.grouped_topk_route(z, correction, top, groups, keep)
 
 
-def routed_combine(ye: torch.Tensor, x: torch.Tensor, rows: torch.Tensor, w: torch.Tensor):
+def routed_combine(
+    ye: torch.Tensor, x: torch.Tensor, rows: Optional[torch.Tensor], w: torch.Tensor,
+    idx: Optional[torch.Tensor] = None, experts: int = 0,
+):
     """out[t] = sum_k w[t, k] * (ye[rows[t, k]] if rows[t, k] >= 0 else x[t]):
     the weighted sum of a token's chosen expert outputs, a negative row
-    standing for an identity expert.  rows int64 [T, top], w fp32 [T, top]."""
+    standing for an identity expert.  rows int64 [T, top], w fp32 [T, top].
+    With rows None every expert saw every token (ye is [experts * T, W],
+    expert-major) and the rows follow from the choices idx int32 [T, top]:
+    idx * T + t, or an identity expert for idx >= experts."""
     T, W = x.shape
     assert ye.dim() == 2 and ye.shape[1] == W and ye.dtype == x.dtype
-    assert rows.dtype == torch.int64 and w.dtype == torch.float32 and rows.shape == w.shape
+    assert w.dtype == torch.float32 and w.dim() == 2
+    if rows is None:
+        assert idx is not None and idx.dtype == torch.int32 and idx.shape == w.shape
+        assert ye.shape[0] == experts * T
+    else:
+        assert rows.dtype == torch.int64 and rows.shape == w.shape
     if _use_hybrid(x):
-        assert ye.is_contiguous() and x.is_contiguous() and rows.is_contiguous() and w.is_contiguous()
+        assert ye.is_contiguous() and x.is_contiguous() and w.is_contiguous()
+        assert (rows if rows is not None else idx).is_contiguous()
         out = torch.empty_like(x)
         _hl().lig_routed_combine(
-            _ptr(out), _ptr(ye), _ptr(x), _ptr(rows), _ptr(w), T, rows.shape[1], W,
-            _is_f32(x), _stream(),
+            _ptr(out), _ptr(ye), _ptr(x), _ptr(rows), _ptr(idx) if rows is None else None,
+            int(experts), _ptr(w), T, w.shape[1], W, _is_f32(x), _stream(),
         )
         return out
+    if rows is None:
+        tok = torch.arange(T, device=x.device).unsqueeze(1)
+        il = idx.long()
+        rows = torch.where(il < experts, il * T + tok, torch.full_like(il, -1))
     return torch_ref.routed_combine(ye, x, rows, w)
 
 

@@ -11,7 +11,10 @@
 //   weights = chosen s / (their sum + 1e-20).
 //
 // routed_combine: out[t] = sum_k w[t, k] * src_k, src_k = ye[row[t, k]] or,
-// for row < 0, the token's own input x[t] (an identity expert).
+// for row < 0, the token's own input x[t] (an identity expert).  Rows come
+// as a table, or are computed from the choices themselves when every expert
+// saw every token (ye = [experts, T, W]): row = idx * T + t, idx >= experts
+// being an identity expert.
 //
 // glu_act over a fused [gate | up] projection:
 //   0: relu(gate) * up
@@ -115,14 +118,22 @@ template <typename T, int N>
 __global__ void routed_combine_kernel(T* __restrict__ out, const T* __restrict__ ye,
                                       const T* __restrict__ x,
                                       const long* __restrict__ rows,
+                                      const int* __restrict__ idx, int experts,
                                       const float* __restrict__ w, int top, int W) {
   const long t = blockIdx.x;
+  const long ntok = gridDim.x;
   for (int c = threadIdx.x * N; c < W; c += blockDim.x * N) {
     float acc[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) acc[i] = 0.f;
     for (int k = 0; k < top; ++k) {
-      const long r = rows[t * top + k];
+      long r;
+      if (idx != nullptr) {
+        const int e = idx[t * top + k];
+        r = e < experts ? (long)e * ntok + t : -1;
+      } else {
+        r = rows[t * top + k];
+      }
       const float wk = w[t * top + k];
       float v[N];
       ldn<N>(r >= 0 ? ye + r * W + c : x + t * W + c, v);
@@ -173,14 +184,14 @@ int lig_grouped_topk_route(const float* z, const float* corr, int T, int N,
 }
 
 void lig_routed_combine(void* out, const void* ye, const void* x, const long* rows,
-                        const float* w, int T, int top, int W, int is_f32,
-                        hipStream_t s) {
+                        const int* idx, int experts, const float* w, int T, int top,
+                        int W, int is_f32, hipStream_t s) {
   if (T <= 0) return;
   const bool v4 = W % 4 == 0 && aligned16(out) && aligned16(ye) && aligned16(x);
   const int threads = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
 #define LIG_RC(T_, N)                                                             \
   hipLaunchKernelGGL((routed_combine_kernel<T_, N>), dim3(T), dim3(threads), 0, s, \
-                     (T_*)out, (const T_*)ye, (const T_*)x, rows, w, top, W)
+                     (T_*)out, (const T_*)ye, (const T_*)x, rows, idx, experts, w, top, W)
   if (is_f32) {
     if (v4) LIG_RC(float, 4); else LIG_RC(float, 1);
   } else {

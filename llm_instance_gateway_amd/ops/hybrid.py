@@ -105,7 +105,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "lig_gelu_erf": [p, p, l, i, p],
         "lig_tanh_act": [p, p, l, i, p],
         "lig_tanh_softcap": [p, f, l, p],
-        "lig_routed_combine": [p, p, p, p, p, i, i, i, i, p],
+        "lig_routed_combine": [p, p, p, p, p, i, p, i, i, i, i, p],
         "lig_glu_act": [p, p, l, i, i, f, f, i, p],
     }
     for name, args in sigs.items():

@@ -302,6 +302,18 @@ def test_routed_combine(device, dtype):
             src = x[t] if rows[t, k] < 0 else ye[rows[t, k]]
             want[t] += w[t, k].item() * src.double().numpy()
     close(got, want, dtype)
+    # every expert saw every token: rows follow from the choices
+    E = 3
+    ye2 = rnd(g, E * T, W).to(dtype)
+    idx = torch.tensor([[0, 2, 4], [3, 1, 0], [2, 2, 2], [5, 4, 3], [1, 0, 2]], dtype=torch.int32)
+    got = ops.routed_combine(ye2.to(device), x.to(device), None, w.to(device), idx=idx.to(device), experts=E)
+    want = np.zeros((T, W))
+    for t in range(T):
+        for k in range(top):
+            e = int(idx[t, k])
+            src = x[t] if e >= E else ye2[e * T + t]
+            want[t] += w[t, k].item() * src.double().numpy()
+    close(got, want, dtype)
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
