@@ -418,27 +418,17 @@ class ScoredExpertsMLP(nn.Module):
             act = ops.silu_mul(torch.bmm(xe.view(E, T, hidden), self.w13).view(E * T, -1))
             ye = torch.bmm(act.view(E, T, self.ff), self.w2)
             return ye.float().sum(dim=0).to(h.dtype)
-        flat_e = idx.reshape(-1)
-        flat_t = torch.arange(T, device=h.device).unsqueeze(1).expand(T, self.top).reshape(-1)
-        order = torch.argsort(flat_e, stable=True)
-        se, stok, sw = flat_e[order], flat_t[order], w.reshape(-1)[order]
-        counts = torch.bincount(se, minlength=E)
-        cap = int(counts.max())  # one host round trip per block; such steps run eager
-        starts = torch.cumsum(counts, 0) - counts
-        pos_in_e = torch.arange(se.numel(), device=h.device) - starts.index_select(0, se)
-        dest = se * cap + pos_in_e
-        gather = torch.full((E * cap,), -1, dtype=torch.int64, device=h.device)
-        gather.index_copy_(0, dest, stok)
+        # (token, expert) pairs into a capacity-padded batch; the chosen score
+        # scales the expert's input row
+        gather, rows, cap = expert_dispatch_plan(idx, E)
         wpad = torch.zeros(E * cap, dtype=torch.float32, device=h.device)
-        wpad.index_copy_(0, dest, sw)
+        wpad.index_copy_(0, rows.reshape(-1), w.reshape(-1))
         xe = ops.scale_gather_rows(h, gather, wpad)
         act = ops.silu_mul(torch.bmm(xe.view(E, cap, hidden), self.w13).view(E * cap, -1))
         ye = torch.bmm(act.view(E, cap, self.ff), self.w2).view(E * cap, hidden)
         # every token owns exactly `top` rows of ye: gather them back in pair
         # order and sum in fp32 (no atomics, the same order every time)
-        back = torch.empty_like(dest)
-        back[order] = dest
-        return ye.index_select(0, back).view(T, self.top, hidden).float().sum(dim=1).to(h.dtype)
+        return ye.index_select(0, rows.reshape(-1)).view(T, self.top, hidden).float().sum(dim=1).to(h.dtype)
 
 
 class NormedRotaryAttention(nn.Module):

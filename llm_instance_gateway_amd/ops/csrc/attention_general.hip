@@ -376,7 +376,7 @@ void lig_paged_attention_general(
     int sigmoid_weights, int gate_per_head, int is_f32, hipStream_t s) {
   if (R <= 0) return;
   // few rows: four waves share each (token, head) so the walk is split
-  const int nw = (long)R * H <= 4096 ? 4 : 1;
+  const int nw = (long)R * H <= 2048 ? 4 : 1;
   dim3 grid(R, H), block(WAVE_SIZE * nw);
   const size_t smem = (size_t)(((D + 1) & ~1) + nw * WAVE_SIZE) * sizeof(float) +
                       (size_t)nw * WAVE_SIZE * sizeof(long) +
