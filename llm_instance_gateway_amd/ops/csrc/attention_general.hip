@@ -2,7 +2,7 @@
 // scores and softmax, gfx950.
 //
 // Serves the shapes the MFMA kernels do not: key size != value size, sizes
-// that are not 64/128, fp32 caches.  One wave per (token, query head) walks
+// that are not 64/128, fp32 caches.  One wave per (token, query head part) walks
 // the sequence's pages 64 keys at a time: lane j scores key j against the
 // query held in LDS, the wave keeps a running max / sum (online softmax),
 // then the lanes switch to value columns and accumulate sum_j p_j V[j, :].
@@ -39,13 +39,18 @@
 
 #define ATT_MAX_DV_PER_LANE 8  // Dv <= 512
 
-// NW waves of a workgroup share one (token, head): wave w takes the 64-key
-// tiles w, w + NW, ... of the walk and keeps its own running max / sum /
-// accumulator; wave 0 merges them through LDS at the end.  Small batches of
+// A wave serves HB query heads of one key/value head at once (HB divides the
+// group size): a key row is loaded once and multiplied with HB queries held in
+// LDS, a value element once and weighted HB times, so grouped-query layers
+// read their cache rows once per group part instead of once per head.
+//
+// NW waves of a workgroup share one (token, head part): wave w takes the
+// 64-key tiles w, w + NW, ... of the walk and keeps its own running max / sum
+// / accumulator; wave 0 merges them through LDS at the end.  Small batches of
 // single tokens, which would otherwise leave most of the chip idle behind one
 // serial walk per wave, run with NW = 4.  Every wave makes the same number of
 // loop trips (a trip without a tile only meets the barriers).
-template <typename T, bool VEC, int NW>
+template <typename T, bool VEC, int NW, int HB>
 __global__ __launch_bounds__(WAVE_SIZE * NW) void paged_attention_general_kernel(
     T* __restrict__ out,  // [R, H * Dv]
     const T* __restrict__ q, long q_stride,
@@ -59,25 +64,25 @@ __global__ __launch_bounds__(WAVE_SIZE * NW) void paged_attention_general_kernel
     const float* __restrict__ score_bias, int sigmoid_weights, int gate_per_head) {
   extern __shared__ __align__(16) float smem[];
   const int Dpad = (D + 1) & ~1;
-  float* q_s = smem;                                   // [D], padded to an even count
-  float* p_all = smem + Dpad;                          // [NW][64]
-  long* voff_all = reinterpret_cast<long*>(p_all + NW * WAVE_SIZE);  // [NW][64]
-  float* ml_s = reinterpret_cast<float*>(voff_all + NW * WAVE_SIZE);  // [NW][2]
-  float* acc_s = ml_s + 2 * NW;                        // [NW][Dv]
+  float* q_s = smem;                                   // [HB][Dpad]
+  float* p_all = smem + HB * Dpad;                     // [NW][HB][64]
+  long* voff_all = reinterpret_cast<long*>(p_all + NW * HB * WAVE_SIZE);  // [NW][64]
+  float* ml_s = reinterpret_cast<float*>(voff_all + NW * WAVE_SIZE);      // [NW][HB][2]
+  float* acc_s = ml_s + 2 * NW * HB;                   // [NW][HB][Dv]
 
-  const int r = blockIdx.x, h = blockIdx.y;
+  const int r = blockIdx.x, h0 = blockIdx.y * HB;
   const int lane = threadIdx.x % WAVE_SIZE, wave = threadIdx.x / WAVE_SIZE;
-  float* p_s = p_all + wave * WAVE_SIZE;
+  float* p_s = p_all + wave * HB * WAVE_SIZE;
   long* voff_s = voff_all + wave * WAVE_SIZE;
   const int seq = tok_seq[r];
-  T* orow = out + (size_t)r * H * Dv + (size_t)h * Dv;
+  T* orow = out + (size_t)r * H * Dv + (size_t)h0 * Dv;  // HB heads side by side
   if (seq < 0) {
-    for (int d = threadIdx.x; d < Dv; d += WAVE_SIZE * NW) st(orow + d, 0.f);
+    for (int d = threadIdx.x; d < HB * Dv; d += WAVE_SIZE * NW) st(orow + d, 0.f);
     return;
   }
   const long pos = positions[r];
   const int ctx = (int)pos + 1;
-  const int g = h / (H / G);
+  const int g = h0 / (H / G);
   const int* bt = block_tables + (size_t)seq * max_blocks;
 
   float tau = 1.f;
@@ -89,23 +94,31 @@ __global__ __launch_bounds__(WAVE_SIZE * NW) void paged_attention_general_kernel
   }
   const float sc = scale * tau;
 
-  const T* qrow = q + (size_t)r * q_stride + (size_t)h * D;
-  for (int d = threadIdx.x; d < D; d += WAVE_SIZE * NW) q_s[d] = ld(qrow + d);
+  const T* qrow = q + (size_t)r * q_stride + (size_t)h0 * D;
+  for (int idx = threadIdx.x; idx < HB * D; idx += WAVE_SIZE * NW) {
+    const int hh = idx / D;
+    q_s[hh * Dpad + (idx - hh * D)] = ld(qrow + idx);
+  }
   __syncthreads();
 
-  float m = -INFINITY, l = 0.f;
-  if (sink != nullptr && wave == 0) {  // the sink is counted once
-    m = sink[h];
-    l = 1.f;
-  }
-  float acc[ATT_MAX_DV_PER_LANE];
+  float m[HB], l[HB], sb[HB];
+  float acc[HB][ATT_MAX_DV_PER_LANE];
 #pragma unroll
-  for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) acc[i] = 0.f;
+  for (int hh = 0; hh < HB; ++hh) {
+    m[hh] = -INFINITY;
+    l[hh] = 0.f;
+    if (sink != nullptr && wave == 0) {  // the sink is counted once
+      m[hh] = sink[h0 + hh];
+      l[hh] = 1.f;
+    }
+    sb[hh] = score_bias != nullptr ? score_bias[h0 + hh] : 0.f;
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) acc[hh][i] = 0.f;
+  }
 
   // chunked visibility: the walk starts at the first key of the query's chunk
   int first_key = chunk > 0 ? (int)(pos / chunk) * chunk : 0;
   if (window > 0) first_key = max(first_key, (int)pos - window + 1);
-  const float sb = score_bias != nullptr ? score_bias[h] : 0.f;
   const int ntiles = (ctx - first_key + WAVE_SIZE - 1) / WAVE_SIZE;
   const int trips = (ntiles + NW - 1) / NW;
   for (int it = 0; it < trips; ++it) {
@@ -114,40 +127,54 @@ __global__ __launch_bounds__(WAVE_SIZE * NW) void paged_attention_general_kernel
     const int j0 = first_key + tile * WAVE_SIZE;
     const int j = j0 + lane;
     const bool valid = active && j < ctx;
-    float score = -INFINITY;
+    float dot[HB];
+#pragma unroll
+    for (int hh = 0; hh < HB; ++hh) dot[hh] = 0.f;
     long voff = 0;
     if (valid) {
       const long blk = bt[j / BS];
       const int off = j % BS;
       const T* krow = k_cache + ((blk * G + g) * BS + off) * (long)D;
       voff = ((blk * G + g) * BS + off) * (long)v_row;
-      float dot = 0.f;
       if (VEC) {  // D % 8 == 0 and 16-byte aligned rows: whole 8-element vectors
         for (int d = 0; d < D; d += 8) {
           float kv[8];
           ld8(krow + d, kv);
 #pragma unroll
-          for (int i = 0; i < 8; ++i) dot += q_s[d + i] * kv[i];
+          for (int hh = 0; hh < HB; ++hh) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dot[hh] += q_s[hh * Dpad + d + i] * kv[i];
+          }
         }
       } else {
-        for (int d = 0; d < D; ++d) dot += q_s[d] * ld(krow + d);
+        for (int d = 0; d < D; ++d) {
+          const float kv = ld(krow + d);
+#pragma unroll
+          for (int hh = 0; hh < HB; ++hh) dot[hh] += q_s[hh * Dpad + d] * kv;
+        }
       }
-      score = dot * sc;
     }
-    float p = 0.f, alpha = 1.f;
-    if (active) {
-      if (sigmoid_weights) {
-        p = valid ? sigmoid_f32(score + sb) : 0.f;
-      } else {
-        const float m_new = fmaxf(m, wave_reduce_max(score));  // finite: key j0 is valid
-        p = valid ? expf(score - m_new) : 0.f;
-        alpha = expf(m - m_new);                               // 0 on the wave's first tile
-        l = l * alpha + wave_reduce_sum(p);
-        m = m_new;
+    float p[HB], alpha[HB];
+#pragma unroll
+    for (int hh = 0; hh < HB; ++hh) {
+      p[hh] = 0.f;
+      alpha[hh] = 1.f;
+      if (active) {
+        const float score = valid ? dot[hh] * sc : -INFINITY;
+        if (sigmoid_weights) {
+          p[hh] = valid ? sigmoid_f32(score + sb[hh]) : 0.f;
+        } else {
+          const float m_new = fmaxf(m[hh], wave_reduce_max(score));  // finite: key j0 is valid
+          p[hh] = valid ? expf(score - m_new) : 0.f;
+          alpha[hh] = expf(m[hh] - m_new);                           // 0 on the wave's first tile
+          l[hh] = l[hh] * alpha[hh] + wave_reduce_sum(p[hh]);
+          m[hh] = m_new;
+        }
       }
     }
     __syncthreads();  // previous tile's readers are done
-    p_s[lane] = p;
+#pragma unroll
+    for (int hh = 0; hh < HB; ++hh) p_s[hh * WAVE_SIZE + lane] = p[hh];
     voff_s[lane] = voff;
     __syncthreads();
     if (active) {
@@ -156,65 +183,82 @@ __global__ __launch_bounds__(WAVE_SIZE * NW) void paged_attention_general_kernel
       for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
         const int d = lane + i * WAVE_SIZE;
         if (d < Dv) {
-          float a = acc[i] * alpha;
-          for (int jj = 0; jj < nv; ++jj) a += p_s[jj] * ld(v_cache + voff_s[jj] + d);
-          acc[i] = a;
+          float a[HB];
+#pragma unroll
+          for (int hh = 0; hh < HB; ++hh) a[hh] = acc[hh][i] * alpha[hh];
+          for (int jj = 0; jj < nv; ++jj) {
+            const float v = ld(v_cache + voff_s[jj] + d);
+#pragma unroll
+            for (int hh = 0; hh < HB; ++hh) a[hh] += p_s[hh * WAVE_SIZE + jj] * v;
+          }
+#pragma unroll
+          for (int hh = 0; hh < HB; ++hh) acc[hh][i] = a[hh];
         }
       }
     }
   }
   if (NW > 1) {
     // wave 0 gathers the other waves' partial results
-    if (lane == 0) {
-      ml_s[2 * wave] = m;
-      ml_s[2 * wave + 1] = l;
-    }
 #pragma unroll
-    for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
-      const int d = lane + i * WAVE_SIZE;
-      if (d < Dv) acc_s[wave * Dv + d] = acc[i];
-    }
-    __syncthreads();
-    if (wave != 0) return;
-    if (sigmoid_weights) {
+    for (int hh = 0; hh < HB; ++hh) {
+      if (lane == 0) {
+        ml_s[2 * (wave * HB + hh)] = m[hh];
+        ml_s[2 * (wave * HB + hh) + 1] = l[hh];
+      }
 #pragma unroll
       for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
         const int d = lane + i * WAVE_SIZE;
-        if (d < Dv)
-          for (int w = 1; w < NW; ++w) acc[i] += acc_s[w * Dv + d];
+        if (d < Dv) acc_s[(wave * HB + hh) * Dv + d] = acc[hh][i];
       }
-    } else {
-      float M = m;  // finite: wave 0 always has the walk's first key
-      for (int w = 1; w < NW; ++w) M = fmaxf(M, ml_s[2 * w]);
-      const float f0 = expf(m - M);
-      l *= f0;
+    }
+    __syncthreads();
+    if (wave != 0) return;
 #pragma unroll
-      for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) acc[i] *= f0;
-      for (int w = 1; w < NW; ++w) {
-        const float fw = expf(ml_s[2 * w] - M);  // 0 for a wave without tiles
-        l += ml_s[2 * w + 1] * fw;
+    for (int hh = 0; hh < HB; ++hh) {
+      if (sigmoid_weights) {
 #pragma unroll
         for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
           const int d = lane + i * WAVE_SIZE;
-          if (d < Dv) acc[i] += acc_s[w * Dv + d] * fw;
+          if (d < Dv)
+            for (int w = 1; w < NW; ++w) acc[hh][i] += acc_s[(w * HB + hh) * Dv + d];
+        }
+      } else {
+        float M = m[hh];  // finite: wave 0 always has the walk's first key
+        for (int w = 1; w < NW; ++w) M = fmaxf(M, ml_s[2 * (w * HB + hh)]);
+        const float f0 = expf(m[hh] - M);
+        l[hh] *= f0;
+#pragma unroll
+        for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) acc[hh][i] *= f0;
+        for (int w = 1; w < NW; ++w) {
+          const float fw = expf(ml_s[2 * (w * HB + hh)] - M);  // 0 for a wave without tiles
+          l[hh] += ml_s[2 * (w * HB + hh) + 1] * fw;
+#pragma unroll
+          for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
+            const int d = lane + i * WAVE_SIZE;
+            if (d < Dv) acc[hh][i] += acc_s[(w * HB + hh) * Dv + d] * fw;
+          }
         }
       }
     }
   }
-  const float inv_l = sigmoid_weights ? 1.f : 1.f / l;
-  float head_gate = 1.f;
-  if (gate != nullptr && gate_per_head)
-    head_gate = sigmoid_f32(ld(gate + (size_t)r * gate_stride + h));
 #pragma unroll
-  for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
-    const int d = lane + i * WAVE_SIZE;
-    if (d < Dv) {
-      float o = acc[i] * inv_l;
-      if (gate_per_head)
-        o *= head_gate;
-      else if (gate != nullptr)
-        o *= sigmoid_f32(ld(gate + (size_t)r * gate_stride + (size_t)h * Dv + d));
-      st(orow + d, o);
+  for (int hh = 0; hh < HB; ++hh) {
+    const int h = h0 + hh;
+    const float inv_l = sigmoid_weights ? 1.f : 1.f / l[hh];
+    float head_gate = 1.f;
+    if (gate != nullptr && gate_per_head)
+      head_gate = sigmoid_f32(ld(gate + (size_t)r * gate_stride + h));
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_DV_PER_LANE; ++i) {
+      const int d = lane + i * WAVE_SIZE;
+      if (d < Dv) {
+        float o = acc[hh][i] * inv_l;
+        if (gate_per_head)
+          o *= head_gate;
+        else if (gate != nullptr)
+          o *= sigmoid_f32(ld(gate + (size_t)r * gate_stride + (size_t)h * Dv + d));
+        st(orow + (size_t)hh * Dv + d, o);
+      }
     }
   }
 }
@@ -375,28 +419,36 @@ void lig_paged_attention_general(
     int v_row, int BS, int chunk, int window, const float* score_bias,
     int sigmoid_weights, int gate_per_head, int is_f32, hipStream_t s) {
   if (R <= 0) return;
-  // few rows: four waves share each (token, head) so the walk is split
-  const int nw = (long)R * H <= 2048 ? 4 : 1;
-  dim3 grid(R, H), block(WAVE_SIZE * nw);
-  const size_t smem = (size_t)(((D + 1) & ~1) + nw * WAVE_SIZE) * sizeof(float) +
+  // heads of one key/value head that a wave serves together
+  const int gs = H / G;
+  const int hb = gs % 4 == 0 ? 4 : (gs % 2 == 0 ? 2 : 1);
+  // few workgroups: four waves share each of them and split the walk
+  const int nw = (long)R * (H / hb) <= 2048 ? 4 : 1;
+  dim3 grid(R, H / hb), block(WAVE_SIZE * nw);
+  const size_t smem = (size_t)(hb * ((D + 1) & ~1) + nw * hb * WAVE_SIZE) * sizeof(float) +
                       (size_t)nw * WAVE_SIZE * sizeof(long) +
-                      (size_t)nw * (2 + Dv) * sizeof(float);
+                      (size_t)nw * hb * (2 + Dv) * sizeof(float);
   const bool vec = D % 8 == 0 && aligned16(k_cache);
-#define LIG_LAUNCH_ATT(T, VEC, NW)                                              \
-  hipLaunchKernelGGL((paged_attention_general_kernel<T, VEC, NW>), grid, block, \
-                     smem, s, (T*)out, (const T*)q, q_stride,                   \
+#define LIG_LAUNCH_ATT(T, VEC, NW, HB)                                          \
+  hipLaunchKernelGGL((paged_attention_general_kernel<T, VEC, NW, HB>), grid,    \
+                     block, smem, s, (T*)out, (const T*)q, q_stride,            \
                      (const T*)k_cache, (const T*)v_cache, block_tables,        \
                      max_blocks, tok_seq, positions, (const T*)gate,            \
                      gate_stride, sink, scale, temp_coef, temp_every,           \
                      temp_every_int, H, G, D, Dv, v_row, BS, chunk, window,      \
                      score_bias, sigmoid_weights, gate_per_head)
+#define LIG_LAUNCH_ATT_H(T, VEC, NW)                    \
+  if (hb == 4) LIG_LAUNCH_ATT(T, VEC, NW, 4);           \
+  else if (hb == 2) LIG_LAUNCH_ATT(T, VEC, NW, 2);      \
+  else LIG_LAUNCH_ATT(T, VEC, NW, 1)
 #define LIG_LAUNCH_ATT_W(T, VEC) \
-  if (nw == 4) LIG_LAUNCH_ATT(T, VEC, 4); else LIG_LAUNCH_ATT(T, VEC, 1)
+  if (nw == 4) { LIG_LAUNCH_ATT_H(T, VEC, 4); } else { LIG_LAUNCH_ATT_H(T, VEC, 1); }
   if (is_f32) {
-    if (vec) { LIG_LAUNCH_ATT_W(float, true); } else { LIG_LAUNCH_ATT_W(float, false); }
+    if (vec) { LIG_LAUNCH_ATT_W(float, true) } else { LIG_LAUNCH_ATT_W(float, false) }
   } else {
-    if (vec) { LIG_LAUNCH_ATT_W(bf16s, true); } else { LIG_LAUNCH_ATT_W(bf16s, false); }
+    if (vec) { LIG_LAUNCH_ATT_W(bf16s, true) } else { LIG_LAUNCH_ATT_W(bf16s, false) }
   }
+#undef LIG_LAUNCH_ATT_H
 #undef LIG_LAUNCH_ATT_W
 #undef LIG_LAUNCH_ATT
 }
