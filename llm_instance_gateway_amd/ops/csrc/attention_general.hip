@@ -419,9 +419,12 @@ void lig_paged_attention_general(
     int v_row, int BS, int chunk, int window, const float* score_bias,
     int sigmoid_weights, int gate_per_head, int is_f32, hipStream_t s) {
   if (R <= 0) return;
-  // heads of one key/value head that a wave serves together
+  // heads of one key/value head that a wave serves together: as many as
+  // divide the group, but fewer while that would leave the chip short of
+  // waves (a small batch of single tokens wants parallel walks first)
   const int gs = H / G;
-  const int hb = gs % 4 == 0 ? 4 : (gs % 2 == 0 ? 2 : 1);
+  int hb = gs % 4 == 0 ? 4 : (gs % 2 == 0 ? 2 : 1);
+  while (hb > 1 && (long)R * (H / hb) * 4 < 2048) hb /= 2;
   // few workgroups: four waves share each of them and split the walk
   const int nw = (long)R * (H / hb) <= 2048 ? 4 : 1;
   dim3 grid(R, H / hb), block(WAVE_SIZE * nw);
