@@ -144,7 +144,9 @@ def test_windowed_attention_rows(device, dtype, kind, window):
     g = torch.Generator().manual_seed(3)
     T, H, G, D, Dv, bs, scale = 150, 4, 2, 12, 6, 16, 0.5
     rows = [149, 148, 130, 128, 127, 112, 100, 80, 65, 64, 63, 49, 48, 16, 15, 7, 6, 1, 0]
-    q, k, v = planted(g, T, H, G, D, Dv, dtype, window_plant(rows, window))
+    # and keys far back (the sequence's first tokens), which only the longest window may see
+    far = [(149, 2), (130, 0), (100, 17)]
+    q, k, v = planted(g, T, H, G, D, Dv, dtype, window_plant(rows, window) + far)
     kc = torch.full((12, G, bs, D), 7.0, dtype=dtype, device=device)
     vc = torch.full((12, G, bs, Dv), -7.0, dtype=dtype, device=device)
     table = [9, 2, 7, 0, 5, 11, 3, 8, 1, 10]
@@ -209,7 +211,8 @@ def test_windowed_attention_prompt_tiles(kind, window, D, Dv):
     qs, gs, wants, tables, at = [], [], [], [], 0
     for ctx, done in seqs:
         rows = [ctx - 1, done, done + 1, min(done + 63, ctx - 1), min(done + 64, ctx - 1), (done + ctx) // 2]
-        q, k, v = planted(g, ctx, H, G, D, Dv, dtype, window_plant(rows, window), boost=4.0)
+        far = [(ctx - 1, 1), (ctx - 1, done)]  # far back, and the portion's first key
+        q, k, v = planted(g, ctx, H, G, D, Dv, dtype, window_plant(rows, window) + far, boost=4.0)
         gate = rnd(g, ctx, H, s=2.0).to(dtype)
         nb = (ctx + bs - 1) // bs
         table = list(range(at, at + nb))[::-1]
